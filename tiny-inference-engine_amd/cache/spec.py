@@ -1,7 +1,10 @@
 """What a mixer needs from the cache, and how a model's needs are grouped.
 
 A mixer declares one need (or none): paged keys and values, all of them or a
-window of them, or a state of fixed size per request. Run-order entries with
+window of them, or a state of fixed size per request; a mixer that keeps several
+things (keys and the last inputs of a short convolution, two mixers side by side)
+declares a tuple of needs and is bound to a tuple of caches in the same order.
+Run-order entries with
 equal needs share a *group*: one page pool, one block table per request and one
 tensor whose leading dimension counts the entries (planes) of the group. The
 reference has a single group - every layer is full attention with the same head
@@ -72,6 +75,10 @@ class FixedState:
 CacheNeed = Union[PagedKV, FixedState]
 
 
+class CallCaches(tuple):
+    """Where a run-order entry whose mixer declared several needs finds them: one ``CallCache`` a need, in order."""
+
+
 @dataclasses.dataclass(frozen=True)
 class CacheGroup:
     need: CacheNeed
@@ -90,7 +97,7 @@ class CallCache:
 @dataclasses.dataclass(frozen=True)
 class CachePlan:
     groups: Tuple[CacheGroup, ...]
-    calls: Tuple[Optional[CallCache], ...]
+    calls: Tuple[Union[None, CallCache, CallCaches], ...]
 
     @functools.cached_property
     def paged_groups(self) -> List[int]:
@@ -104,7 +111,8 @@ class CachePlan:
 def plan_cache(needs: Sequence[Optional[CacheNeed]], reads_cache_of: Sequence[Optional[int]]) -> CachePlan:
     """Groups the needs of the run-order entries.
 
-    ``needs[i]`` is what entry i's mixer needs (None for a mixer without cache);
+    ``needs[i]`` is what entry i's mixer needs (None for a mixer without cache, a tuple for
+    a mixer that needs several things: its entry of ``calls`` is then a ``CallCaches``);
     ``reads_cache_of[i]`` is an earlier entry whose plane entry i reads instead
     of owning one, and whose need must equal its own.
     """
@@ -112,29 +120,37 @@ def plan_cache(needs: Sequence[Optional[CacheNeed]], reads_cache_of: Sequence[Op
         raise InvalidArgument("plan_cache: one need and one sharing entry per run-order entry")
     group_of = {}
     planes: List[int] = []
-    calls: List[Optional[CallCache]] = []
-    for i, need in enumerate(needs):
-        src = reads_cache_of[i]
-        if need is None:
-            if src is not None:
-                raise InvalidArgument(f"run order entry {i} reads a cache but its mixer needs none")
-            calls.append(None)
-            continue
-        if src is not None:
-            owner = calls[src] if 0 <= src < i else None
-            if owner is None or not owner.writes:
-                raise InvalidArgument(f"run order entry {i} reads the cache of entry {src}, which owns none")
-            if needs[src] != need:
-                raise InvalidArgument(
-                    f"run order entry {i} needs {need} but reads the cache of entry {src}, which holds {needs[src]}")
-            calls.append(CallCache(owner.group, owner.plane, False))
-            continue
+    calls: List[Union[None, CallCache, CallCaches]] = []
+
+    def own(need) -> CallCache:
         if need not in group_of:
             group_of[need] = len(planes)
             planes.append(0)
         g = group_of[need]
-        calls.append(CallCache(g, planes[g], True))
         planes[g] += 1
+        return CallCache(g, planes[g] - 1, True)
+
+    for i, need in enumerate(needs):
+        src = reads_cache_of[i]
+        if need is None or (isinstance(need, (tuple, list)) and not need):
+            if src is not None:
+                raise InvalidArgument(f"run order entry {i} reads a cache but its mixer needs none")
+            calls.append(None)
+            continue
+        several = isinstance(need, (tuple, list))
+        if src is not None:
+            owner = calls[src] if 0 <= src < i else None
+            owners = owner if isinstance(owner, CallCaches) else (owner,)
+            if owner is None or not all(o.writes for o in owners):
+                raise InvalidArgument(f"run order entry {i} reads the cache of entry {src}, which owns none")
+            theirs = needs[src]
+            if (tuple(theirs) if isinstance(theirs, (tuple, list)) else theirs) != (tuple(need) if several else need):
+                raise InvalidArgument(
+                    f"run order entry {i} needs {need} but reads the cache of entry {src}, which holds {needs[src]}")
+            read = [CallCache(o.group, o.plane, False) for o in owners]
+            calls.append(CallCaches(read) if several else read[0])
+            continue
+        calls.append(CallCaches(own(n) for n in need) if several else own(need))
     ordered = sorted(group_of.items(), key=lambda kv: kv[1])
     groups = tuple(CacheGroup(need, planes[g]) for need, g in ordered)
     return CachePlan(groups, tuple(calls))

@@ -62,6 +62,15 @@ __device__ __forceinline__ float tanh_fast(float x) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
 }
 
+// The tanh form of gelu, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), with the library's tanhf (float32 paths)
+// and with tanh_fast (epilogues of the bfloat16 products, whose results are rounded to 8 bits of mantissa anyway).
+__device__ __forceinline__ float gelu_tanh_exact(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float gelu_tanh_fast(float z) {
+  return 0.5f * z * (1.0f + tanh_fast(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
 // The first key a query at position pos reads: every key (0), the last `window` ones, or those of its own
 // chunk of `chunk` positions counted from position 0 of the sequence. At most one of the two is positive.
 __device__ __forceinline__ int first_visible_key(int pos, int window, int chunk) {

@@ -159,7 +159,8 @@ extern "C" int tie_rms_norm(const void* x, int x_dtype, const float* w, float ep
 // ------------------------------------------------------------------- SwiGLU
 // gate_up is [T, 2I] with the gate in columns [0, I) and up in [I, 2I).
 // out[t, i] = gate / (1 + exp(-gate)) * up, left to right. Reference: cpu_backend.cpp:195-207.
-template <typename TX, typename TO>
+// ACT 0: the gate goes through silu; 1: through the tanh form of gelu (gate_activation of common.h).
+template <typename TX, typename TO, int ACT>
 __global__ void swiglu_kernel(const TX* __restrict__ gate_up, TO* __restrict__ out, int I) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -167,19 +168,22 @@ __global__ void swiglu_kernel(const TX* __restrict__ gate_up, TO* __restrict__ o
   const TX* row = gate_up + static_cast<size_t>(t) * 2 * I;
   const float g = load_as_float(row + i);
   const float u = load_as_float(row + I + i);
-  store_from_float(out + static_cast<size_t>(t) * I + i, g / (1.0f + expf(-g)) * u);
+  store_from_float(out + static_cast<size_t>(t) * I + i, (ACT == 0 ? g / (1.0f + expf(-g)) : gelu_tanh_exact(g)) * u);
 }
 
-extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int T, int I,
+extern "C" int tie_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int T, int I, int activation,
                           hipStream_t stream) {
-  if (T <= 0 || I <= 0 || T > 65535 * 64) return TIE_BAD_ARGUMENT;
+  if (T <= 0 || I <= 0 || T > 65535 * 64 || activation < 0 || activation > 1) return TIE_BAD_ARGUMENT;
   const dim3 grid((I + 255) / 256, T);
-#define LAUNCH(TX, TO) \
-  swiglu_kernel<TX, TO><<<grid, 256, 0, stream>>>(static_cast<const TX*>(gate_up), static_cast<TO*>(out), I)
-  if (in_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float);
-  else if (in_dtype == TIE_F32 && out_dtype == TIE_BF16) LAUNCH(float, bf16_t);
-  else if (in_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t);
-  else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(bf16_t, float);
+#define LAUNCH(TX, TO)                                                                                             \
+  if (activation == 0)                                                                                             \
+    swiglu_kernel<TX, TO, 0><<<grid, 256, 0, stream>>>(static_cast<const TX*>(gate_up), static_cast<TO*>(out), I); \
+  else                                                                                                             \
+    swiglu_kernel<TX, TO, 1><<<grid, 256, 0, stream>>>(static_cast<const TX*>(gate_up), static_cast<TO*>(out), I)
+  if (in_dtype == TIE_F32 && out_dtype == TIE_F32) { LAUNCH(float, float); }
+  else if (in_dtype == TIE_F32 && out_dtype == TIE_BF16) { LAUNCH(float, bf16_t); }
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_BF16) { LAUNCH(bf16_t, bf16_t); }
+  else if (in_dtype == TIE_BF16 && out_dtype == TIE_F32) { LAUNCH(bf16_t, float); }
   else return TIE_BAD_ARGUMENT;
 #undef LAUNCH
   return tie_launch_status();
@@ -728,23 +732,25 @@ __global__ __launch_bounds__(QK4_THREADS) void qk_norm_rope_kv_write4_kernel(
 }
 
 // angles[t, 0:Dh/2] = cos(float(positions[t]) * inv_freq[i]), angles[t, Dh/2:Dh] = sin of the same: what
-// the kernel below would compute per head and layer, once per step instead.
+// the kernel below would compute per head and layer, once per step instead. Both are multiplied by `amplitude`
+// (1 for a plain rotation; encodings that stretch the frequencies for longer contexts scale the rotated pair).
 __global__ void rope_angles_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                   float* __restrict__ angles, int T, int half) {
+                                   float* __restrict__ angles, int T, int half, float amplitude) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= T * half) return;
   const int t = i / half, p = i % half;
   float sn, cs;
   sincosf(static_cast<float>(positions[t]) * inv_freq[p], &sn, &cs);
-  angles[static_cast<size_t>(t) * 2 * half + p] = cs;
-  angles[static_cast<size_t>(t) * 2 * half + half + p] = sn;
+  angles[static_cast<size_t>(t) * 2 * half + p] = cs * amplitude;
+  angles[static_cast<size_t>(t) * 2 * half + half + p] = sn * amplitude;
 }
 
 extern "C" int tie_rope_angles(const int* positions, const float* inv_freq, float* angles, int T, int half,
-                               hipStream_t stream) {
+                               float amplitude, hipStream_t stream) {
   if (T <= 0 || half <= 0) return TIE_BAD_ARGUMENT;
   const long n = static_cast<long>(T) * half;
-  rope_angles_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, stream>>>(positions, inv_freq, angles, T, half);
+  rope_angles_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, stream>>>(positions, inv_freq, angles, T, half,
+                                                                                 amplitude);
   return tie_launch_status();
 }
 

@@ -73,6 +73,7 @@ __device__ __forceinline__ void store_slice(bf16_t* lds, const uint4 (&regs)[ROW
 // EPI: 0 = store float32, 1 = store bfloat16, 2 = add to float32 output,
 //      3 = gated: columns come in blocks of 16 = 8 gate columns then 8 up columns of the same 8 outputs;
 //          out[m, block * 8 + j] = silu(gate_j) * up_j as bfloat16, out has N / 2 columns
+//      4 = the same with the tanh form of gelu on the gate
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int EPI>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const bf16_t* __restrict__ x_all,
                                                                           const bf16_t* __restrict__ w_all,
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int m = row0 + wm * WM + i * 32 + 8 * (v / 4) + fk * 4 + (v % 4);
-        if (EPI == 3) {
+        if (EPI == 3 || EPI == 4) {
           // The partner column (gate <-> up) sits 8 lanes away; every lane takes part in the exchange.
           const float mine = acc[i][j][v];
           const float other = __shfl_xor(mine, 8, 64);
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_bf16_kernel(const 
             const float g = mine, u = other;
             const int out_col = (n >> 4) * 8 + (n & 7);
             static_cast<bf16_t*>(outp)[static_cast<size_t>(m) * (N / 2) + out_col] =
-                float_to_bf16(g / (1.0f + __expf(-g)) * u);
+                float_to_bf16((EPI == 4 ? gelu_tanh_fast(g) : g / (1.0f + __expf(-g))) * u);
           }
           continue;
         }
@@ -284,7 +285,7 @@ static int launch_gemm(const void* x, const void* w, void* out, int epi, int M, 
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n,        \
         per_split);                                                                                          \
   }
-  if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
+  if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else if (epi == 3) LAUNCH(3) else LAUNCH(4)
 #undef LAUNCH
   return tie_launch_status();
 }
@@ -518,7 +519,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
   }
   for (; kt < k_tiles; ++kt) slice(kt, std::false_type{});
 
-  const bool gated_n = EPI == 3;
+  const bool gated_n = EPI == 3 || EPI == 4;
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int m = row0 + wm * (BM / 2) + i * 32 + fr;
@@ -538,8 +539,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                       u3 = acc[i][j][4 * g + 7];
           const int out_col = (n >> 4) * 8 + 4 * fk;
           uint2 pk;
-          pk.x = pack_bf16x2(v0 / (1.0f + __expf(-v0)) * u0, v1 / (1.0f + __expf(-v1)) * u1);
-          pk.y = pack_bf16x2(v2 / (1.0f + __expf(-v2)) * u2, v3 / (1.0f + __expf(-v3)) * u3);
+          if (EPI == 4) {
+            pk.x = pack_bf16x2(gelu_tanh_fast(v0) * u0, gelu_tanh_fast(v1) * u1);
+            pk.y = pack_bf16x2(gelu_tanh_fast(v2) * u2, gelu_tanh_fast(v3) * u3);
+          } else {
+            pk.x = pack_bf16x2(v0 / (1.0f + __expf(-v0)) * u0, v1 / (1.0f + __expf(-v1)) * u1);
+            pk.y = pack_bf16x2(v2 / (1.0f + __expf(-v2)) * u2, v3 / (1.0f + __expf(-v3)) * u3);
+          }
           *reinterpret_cast<uint2*>(static_cast<bf16_t*>(outp) + static_cast<size_t>(m) * (N / 2) + out_col) = pk;
           continue;
         }
@@ -584,7 +590,7 @@ static int launch_gemm_dma(const void* x, const void* w, void* out, int epi, int
     gemm_bf16_dma_kernel<BM, BN, EPI, PW><<<grid, 256, shared, stream>>>(                                    \
         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), out, M, N, K, tiles_m, tiles_n, per_split); \
   }
-  if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else LAUNCH(3)
+  if (epi == 0) LAUNCH(0) else if (epi == 1) LAUNCH(1) else if (epi == 2) LAUNCH(2) else if (epi == 3) LAUNCH(3) else LAUNCH(4)
 #undef LAUNCH
   return tie_launch_status();
 }
@@ -786,7 +792,7 @@ extern "C" int tie_gemm_bf16(const void* x, const void* w, void* out, int out_dt
   if (out_dtype != TIE_F32 && out_dtype != TIE_BF16) return TIE_BAD_ARGUMENT;
   if (gated && (accumulate || out_dtype != TIE_BF16 || N % 16 != 0)) return TIE_BAD_ARGUMENT;
   if (splits > 1 && (accumulate || gated || out_dtype != TIE_F32)) return TIE_BAD_ARGUMENT;
-  const int epi = gated ? 3 : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
+  const int epi = gated ? (gated == 2 ? 4 : 3) : (accumulate ? 2 : (out_dtype == TIE_F32 ? 0 : 1));
   const bool straight = gemm_dma_takes(x, w, out, N, K, splits);
   if (packed && (N % 16 != 0 || !straight || (tile != 0 && (tile < 4 || tile > 10)))) return TIE_BAD_ARGUMENT;
   if (tile == 0) {

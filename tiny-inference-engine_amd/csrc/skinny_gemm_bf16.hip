@@ -318,7 +318,7 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_gemm_kernel(const bf16
 #pragma unroll
       for (int wv = 1; wv < WAVES; ++wv) up += red[wv][mt][t][ee + 8];
       if (scaled) up *= row_scale;
-      store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, sum / (1.0f + __expf(-sum)) * up);
+      store_from_float(out + static_cast<size_t>(m) * (N / 2) + (n0 + t * 16) / 2 + c, (gated == 2 ? gelu_tanh_fast(sum) : sum / (1.0f + __expf(-sum))) * up);
       continue;
     }
     TO* o = out + (static_cast<size_t>(partial ? split : 0) * M + m) * N + n;
@@ -511,7 +511,7 @@ __global__ __launch_bounds__(WAVES* TIE_WAVE) void skinny_rows_kernel(const bf16
         if (gated) {       // columns 0..7 are gates, 8..15 the ups of the same outputs
           const float up = __shfl(sum, (lane & 48) | ((c + 8) & 15), TIE_WAVE);
           if (m < M && c < 8)
-            store_from_float(out + static_cast<size_t>(m) * (N / 2) + (tile0 + t) * 8 + c, sum / (1.0f + __expf(-sum)) * up);
+            store_from_float(out + static_cast<size_t>(m) * (N / 2) + (tile0 + t) * 8 + c, (gated == 2 ? gelu_tanh_fast(sum) : sum / (1.0f + __expf(-sum))) * up);
           continue;
         }
         if (m >= M) continue;
@@ -662,7 +662,7 @@ extern "C" int tie_skinny_norm_epilogue_rows(int N, int K) {
 }
 
 // gated: w holds blocks of 16 rows = 8 gate rows then 8 up rows of the same 8 outputs; out has N / 2 columns
-// and receives silu(gate) * up.
+// and receives silu(gate) * up (gated == 1) or gelu_tanh(gate) * up (gated == 2).
 // splits > 1: out is float32 [splits, M, N], plane s holding the sums over the s-th range of K.
 // packed: w is in the blocked layout described at the top (N % 16 == 0 and K % 32 == 0).
 static int launch_skinny(const void* x, const void* w, void* out, int out_dtype, int accumulate, int gated, int M,

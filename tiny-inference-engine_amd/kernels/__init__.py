@@ -58,6 +58,9 @@ _SOURCES = {
     "machine_peaks": ("tie_machine_peaks", "machine_peaks.hip"),
     "moe": ("tie_moe", "moe.hip"),
     "recurrent": ("tie_recurrent", "recurrent.hip"),
+    "hyper": ("tie_hyper", "hyper.hip"),
+    "delta_rule": ("tie_delta_rule", "delta_rule.hip"),
+    "latent": ("tie_latent", "latent.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -83,13 +86,13 @@ _SIGNATURES = {
         "tie_poly_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_scale_softcap": [_c_void, ctypes.c_longlong, _c_float, _c_float, _c_void],
         "tie_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
-        "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
+        "tie_swiglu": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
         "tie_cast": [_c_void, _c_int, _c_void, _c_int, ctypes.c_longlong, _c_void],
         "tie_scale_rows": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_float, _c_float, _c_void],
         "tie_add_bias": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_void],
         "tie_take_tokens": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
         "tie_random_fill": [_c_void, ctypes.c_longlong, ctypes.c_ulonglong, _c_int, ctypes.c_double, _c_void],
-        "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_rope_angles": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_float, _c_void],
         "tie_qk_norm_rope_kv_write": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_float, _c_void, _c_void,
                                       _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void, _c_int, _c_int,
                                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_long, _c_int, _c_int, _c_int,
@@ -131,6 +134,29 @@ _SIGNATURES = {
         "tie_gated_rms_norm": [_c_void, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
         "tie_min_gru_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void,
                              _c_void, _c_int, _c_void, _c_void, _c_void],
+    },
+    "hyper": {
+        "tie_layer_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int, _c_void],
+        "tie_hyper_connection": [_c_void, _c_long, _c_int, _c_int, _c_void, _c_int, _c_void, _c_long, _c_int, _c_void,
+                                 _c_void, _c_void, _c_void, _c_float, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
+    },
+    "delta_rule": {
+        "tie_conv_qkv": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int,
+                         _c_int, _c_void, _c_void, _c_float, _c_float, _c_float, _c_void, _c_int, _c_void],
+        "tie_conv_state_update": [_c_void, _c_int, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
+        "tie_delta_prepare": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int,
+                              _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void],
+        "tie_gated_delta_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int,
+                                 _c_int, _c_int, _c_void],
+        "tie_grouped_gated_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int,
+                                       _c_int, _c_int, _c_void],
+    },
+    "latent": {
+        "tie_latent_prepare": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
+                               _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                               _c_int, _c_void],
+        "tie_head_linear": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void,
+                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void],
     },
     "skinny_gemm_bf16": {
         "tie_skinny_gemm_splits": [_c_int, _c_int],
@@ -390,15 +416,22 @@ def add_partials(x: torch.Tensor, partials: torch.Tensor, weight: Optional[torch
         _stream())
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up of shape [T, 2I]."""
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i] for gate_up of shape [T, 2I]; ``activation`` "silu" or
+    "gelu_tanh" (``0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))``)."""
+    if activation not in GATE_ACTIVATIONS:
+        raise InvalidArgument(f"a gate's activation is one of {', '.join(GATE_ACTIVATIONS)}, not '{activation}'")
     _gpu(gate_up, "swiglu input")
     _gpu(out, "swiglu output")
     T, two_i = gate_up.shape
     if two_i % 2 or tuple(out.shape) != (T, two_i // 2):
         raise InvalidArgument(f"swiglu: input {list(gate_up.shape)} and output {list(out.shape)} do not match")
     _call(_lib("elementwise").tie_swiglu, "swiglu", gate_up.data_ptr(), _code(gate_up, "swiglu input"), out.data_ptr(),
-                                          _code(out, "swiglu output"), T, two_i // 2, _stream())
+                                          _code(out, "swiglu output"), T, two_i // 2, GATE_ACTIVATIONS[activation],
+                                          _stream())
 
 
 def gelu(x: torch.Tensor, out: torch.Tensor) -> None:
@@ -800,15 +833,17 @@ def decode_product_rows(M: int, w, gated: bool = False) -> bool:
 
 
 def linear_swiglu(x: torch.Tensor, w_interleaved: torch.Tensor, out: torch.Tensor,
-                  row_scale: Optional[RowScale] = None) -> None:
-    """out = silu(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only.
-    ``row_scale`` as in ``skinny_gemm_bf16`` (up to ``NORM_EPILOGUE_ROWS`` rows)."""
+                  row_scale: Optional[RowScale] = None, activation: str = "silu") -> None:
+    """out = act(x @ gate.T) * (x @ up.T) in one product over the interleaved weight; bfloat16 only.
+    ``row_scale`` as in ``skinny_gemm_bf16`` (up to ``NORM_EPILOGUE_ROWS`` rows); ``activation`` "silu" or
+    "gelu_tanh"."""
+    gated = 1 + GATE_ACTIVATIONS[activation]
     if decode_product_rows(x.shape[0], w_interleaved, gated=True):
-        skinny_gemm_bf16(x, w_interleaved, out, gated=True, row_scale=row_scale)
+        skinny_gemm_bf16(x, w_interleaved, out, gated=gated, row_scale=row_scale)
     elif row_scale is not None:
         raise InvalidArgument(f"{x.shape[0]} rows without their norm's factor: only the decode product applies it")
     else:
-        gemm_bf16(x, w_interleaved, out, gated=True)
+        gemm_bf16(x, w_interleaved, out, gated=gated)
 
 
 @functools.lru_cache(maxsize=None)
@@ -846,15 +881,16 @@ def linear(x: torch.Tensor, w, out: torch.Tensor, accumulate: bool = False, row_
         gemm_generic(x, w, out, accumulate)
 
 
-def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t] = [cos(float(positions[t]) * inv_freq), sin(...)]: the rotation table of one step, ``[T, 2 * half]`` float32."""
+def rope_angles(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor, amplitude: float = 1.0) -> None:
+    """out[t] = amplitude * [cos(float(positions[t]) * inv_freq), sin(...)]: the rotation table of one step,
+    ``[T, 2 * half]`` float32."""
     T = positions.numel()
     half = inv_freq.numel()
     _i32(positions, "positions", T)
     _f32(inv_freq, "inv_freq", (half,))
     _f32(out, "rope angles", (T, 2 * half))
     _call(_lib("elementwise").tie_rope_angles, "rope_angles", positions.data_ptr(), inv_freq.data_ptr(), out.data_ptr(), T, half,
-                                               _stream())
+                                               float(amplitude), _stream())
 
 
 def qk_norm_rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, q_weight: Optional[torch.Tensor],
@@ -1843,3 +1879,282 @@ def moe_combine(routed: RoutedParts, out: torch.Tensor, accumulate: bool = False
     _call(_lib("moe").tie_moe_combine, "moe_combine", routed.parts.data_ptr(), routed.where.data_ptr(),
           routed.weights.data_ptr(), routed.self_rows.data_ptr(), _code(routed.self_rows, "input rows"),
           out.data_ptr(), T, top, n, int(accumulate), _stream())
+
+
+# ------------------------------------------------- layer norm, hyper-connections
+HYPER_MAX_STREAMS = 8        # HYPER_MAX_STREAMS of csrc/hyper.hip
+ROW_IN_LDS_MAX = 16384       # the widest row the kernels that keep a float32 row in LDS take
+_NORM_KINDS = {"layer_norm": 0, "rms_norm": 1, None: 2}
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+               rows: Optional[torch.Tensor] = None) -> None:
+    """out = (x - mean) / sqrt(var + eps) * weight row by row (no bias; the variance is the mean of the squared
+    deviations; float32 statistics). ``rows`` (int32) picks the rows of ``x`` that are normed."""
+    _gpu(x, "layer norm input")
+    _gpu(out, "layer norm output")
+    n = x.shape[-1]
+    count = x.shape[0] if rows is None else rows.numel()
+    _f32(weight, "layer norm weight", (n,))
+    if x.dim() != 2 or tuple(out.shape) != (count, n) or n > ROW_IN_LDS_MAX:
+        raise InvalidArgument(f"layer norm: input {list(x.shape)} / output {list(out.shape)} do not fit {count} rows "
+                              f"of at most {ROW_IN_LDS_MAX}")
+    if rows is not None:
+        _i32(rows, "row indices")
+    if count == 0:
+        return
+    _call(_lib("hyper").tie_layer_norm, "layer_norm", x.data_ptr(), _code(x, "layer norm input"), weight.data_ptr(),
+          float(eps), out.data_ptr(), _code(out, "layer norm output"), _ptr(rows), count, n, _stream())
+
+
+def hyper_connection(streams: torch.Tensor, x: Optional[torch.Tensor] = None, from_x: bool = False, fold: bool = False,
+                     write: Optional[tuple] = None, read: Optional[tuple] = None) -> None:
+    """One pass over the residual streams ``[S, T, n]`` (float32) of a model with hyper-connections.
+
+    ``write`` ``(y, mix, out)``: every stream t becomes ``sum_s mix[s, t] * stream_s + out[t] * y`` from the old
+    streams; ``y`` is float32 rows ``[T, n]`` or planes of partial sums ``[P, T, n]`` added in plane order.
+    ``from_x``: the streams do not exist yet; all equal the rows of ``x`` (and are stored). ``fold``: ``x`` receives
+    the sum of the (new) streams. ``read`` ``(in, norm_kind, weight, eps, h)``: ``h = norm(sum_s in[s] * stream_s)``
+    of the new streams, ``norm_kind`` "layer_norm", "rms_norm" or None (``h`` is then the float32 sum itself)."""
+    _f32(streams, "residual streams")
+    if streams.dim() != 3 or streams.shape[0] > HYPER_MAX_STREAMS:
+        raise InvalidArgument(f"residual streams {list(streams.shape)} must be [streams <= {HYPER_MAX_STREAMS}, rows, width]")
+    S, T, n = streams.shape
+    if n > ROW_IN_LDS_MAX:
+        raise InvalidArgument(f"rows of {n} exceed the {ROW_IN_LDS_MAX} this kernel takes")
+    if from_x or fold:
+        _f32(x, "the residual rows", (T, n))
+    y = mix = out_w = None
+    planes, plane_stride = 0, 0
+    if write is not None:
+        y, mix, out_w = write
+        _f32(y, "the sub-layer's result")
+        if y.dim() == 2:
+            y = y.unsqueeze(0)
+        if tuple(y.shape[1:]) != (T, n):
+            raise InvalidArgument(f"a sub-layer's result {list(y.shape)} does not fit {T} rows of {n}")
+        planes, plane_stride = y.shape[0], y.stride(0)
+        _f32(mix, "stream mixing weights", (S, S))
+        _f32(out_w, "stream output weights", (S,))
+    in_w = w = h = None
+    eps, kind, h_code = 0.0, 2, F32
+    if read is not None:
+        in_w, norm_kind, w, eps, h = read
+        _f32(in_w, "stream input weights", (S,))
+        kind = _NORM_KINDS[norm_kind]
+        _gpu(h, "normed rows")
+        if tuple(h.shape) != (T, n) or (kind == 2 and h.dtype != torch.float32):
+            raise InvalidArgument(f"normed rows {list(h.shape)} {h.dtype} do not fit {[T, n]}")
+        if kind != 2:
+            _f32(w, "norm weight", (n,))
+        h_code = _code(h, "normed rows")
+    if T == 0:
+        return
+    _call(_lib("hyper").tie_hyper_connection, "hyper_connection", streams.data_ptr(), streams.stride(0), S, int(from_x),
+          _ptr(x), int(fold), _ptr(y), plane_stride, planes, _ptr(mix), _ptr(out_w), _ptr(in_w), _ptr(w), float(eps),
+          kind, _ptr(h), h_code, T, n, _stream())
+
+
+# ------------------------------------------------- short convolutions, the gated delta rule
+CONV_MAX_TAPS = 8            # CONV_MAX_TAPS of csrc/delta_rule.hip
+DELTA_RULE_MAX_DIM = 256     # key rows of a state the scan kernel keeps in registers (a quarter of them a wave)
+
+
+def conv_qkv(u: torch.Tensor, weight: torch.Tensor, taps: int, state: Optional[torch.Tensor], batch, sizes,
+             out: torch.Tensor, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+             counts=None, eps: float = 0.0) -> None:
+    """The short causal convolution of an attention's projected q, k and v, and the norms over a whole projection.
+
+    ``u``: float32 rows ``[T, >= nq + nk + nv]``, ``sizes`` = ``(nq, nk, nv)``; ``weight`` float32 ``[C, taps]``
+    (the last tap is the current token's); ``state`` ``[slots, taps - 1, C]`` holds every sequence's last inputs
+    (read here; ``conv_state_update`` writes it). ``q_norm`` / ``k_norm`` (float32 ``[nq]`` / ``[nk]``): q and k are
+    divided by their root mean square over all heads at once (over ``counts`` = (values of q, of k) where fewer than
+    the columns count) and multiplied by these. ``out``: float32 ``[T, C]`` rows."""
+    nq, nk, nv = (int(v) for v in sizes)
+    C = nq + nk + nv
+    _gpu_strided(u, "projected rows")
+    T = u.shape[0]
+    if u.dtype != torch.float32 or u.dim() != 2 or u.shape[1] < C or u.stride(1) != 1:
+        raise InvalidArgument(f"projected rows {list(u.shape)} {u.dtype} do not hold {C} float32 columns")
+    _f32(weight, "convolution weights", (C, taps))
+    _gpu_strided(out, "convolved rows")
+    if out.dtype != torch.float32 or tuple(out.shape) != (T, C) or out.stride(1) != 1:
+        raise InvalidArgument(f"convolved rows {list(out.shape)} do not fit {[T, C]}")
+    if not 1 <= taps <= CONV_MAX_TAPS or C > ROW_IN_LDS_MAX:
+        raise InvalidArgument(f"a convolution of {taps} taps over {C} channels exceeds {CONV_MAX_TAPS} taps or "
+                              f"{ROW_IN_LDS_MAX} channels")
+    if taps > 1:
+        _f32(state, "convolution state")
+        if tuple(state.shape[1:]) != (taps - 1, C):
+            raise InvalidArgument(f"convolution state {list(state.shape)} does not fit {[taps - 1, C]} a slot")
+    if q_norm is not None:
+        _f32(q_norm, "q norm weight", (nq,))
+    if k_norm is not None:
+        _f32(k_norm, "k norm weight", (nk,))
+    count_q, count_k = counts if counts is not None else (nq, nk)
+    if T == 0:
+        return
+    _call(_lib("delta_rule").tie_conv_qkv, "conv_qkv", u.data_ptr(), u.stride(0), weight.data_ptr(), taps, _ptr(state),
+          batch.state_slots.data_ptr(), batch.seq_of_row.data_ptr(), batch.query_start.data_ptr(), T, nq, nk, nv,
+          _ptr(q_norm), _ptr(k_norm), float(count_q), float(count_k), float(eps), out.data_ptr(), out.stride(0),
+          _stream())
+
+
+def conv_state_update(u: torch.Tensor, taps: int, state: torch.Tensor, batch, channels: int) -> None:
+    """After a step: every sequence's slot of ``state`` ``[slots, taps - 1, C]`` holds its last ``taps - 1`` inputs
+    (rows of ``u``, or what the state held where the step brought fewer)."""
+    if taps <= 1:
+        return
+    _gpu_strided(u, "projected rows")
+    _f32(state, "convolution state")
+    if u.dtype != torch.float32 or u.shape[1] < channels or tuple(state.shape[1:]) != (taps - 1, channels):
+        raise InvalidArgument(f"rows {list(u.shape)} / state {list(state.shape)} do not fit {channels} channels, {taps} taps")
+    if batch.num_seqs == 0:
+        return
+    _call(_lib("delta_rule").tie_conv_state_update, "conv_state_update", u.data_ptr(), u.stride(0), taps,
+          state.data_ptr(), batch.state_slots.data_ptr(), batch.query_start.data_ptr(), batch.num_seqs, channels,
+          _stream())
+
+
+def delta_prepare(u: torch.Tensor, weight: torch.Tensor, taps: int, state: Optional[torch.Tensor], batch,
+                  a: torch.Tensor, A_log: torch.Tensor, dt_bias: torch.Tensor, kv_heads: int, heads: int, key_dim: int,
+                  value_dim: int, out: torch.Tensor) -> None:
+    """What the gated delta rule takes of every token, from the projections' float32 sums.
+
+    ``u`` rows ``[q (G d) | k (G d) | v (H e) | b (H)]``: q, k, v through the short convolution and silu, q and k
+    made unit vectors per head (q also times ``d ** -0.5``), ``beta = sigmoid(b)``; ``a`` rows ``[H d]``: the decays
+    ``exp(-exp(A_log[head]) * softplus(a + dt_bias))``. ``out`` rows: ``[q | k | v | beta | decay]`` float32."""
+    G, H, d, e = kv_heads, heads, key_dim, value_dim
+    C = 2 * G * d + H * e
+    _gpu_strided(u, "projected rows")
+    _gpu_strided(a, "decay rows")
+    T = u.shape[0]
+    if u.dtype != torch.float32 or u.shape[1] < C + H or a.dtype != torch.float32 or tuple(a.shape) != (T, H * d):
+        raise InvalidArgument(f"projected rows {list(u.shape)} / decay rows {list(a.shape)} do not fit the heads")
+    _f32(weight, "convolution weights", (C, taps))
+    _f32(A_log, "A_log", (H,))
+    _f32(dt_bias, "dt_bias", (H * d,))
+    _f32(out, "delta rule rows", (T, C + H + H * d))
+    if not 1 <= taps <= CONV_MAX_TAPS or C > ROW_IN_LDS_MAX:
+        raise InvalidArgument(f"a convolution of {taps} taps over {C} channels exceeds what the kernel takes")
+    if taps > 1:
+        _f32(state, "convolution state")
+        if tuple(state.shape[1:]) != (taps - 1, C):
+            raise InvalidArgument(f"convolution state {list(state.shape)} does not fit {[taps - 1, C]} a slot")
+    if T == 0:
+        return
+    _call(_lib("delta_rule").tie_delta_prepare, "delta_prepare", u.data_ptr(), u.stride(0), weight.data_ptr(), taps,
+          _ptr(state), batch.state_slots.data_ptr(), batch.seq_of_row.data_ptr(), batch.query_start.data_ptr(),
+          a.data_ptr(), a.stride(0), A_log.data_ptr(), dt_bias.data_ptr(), T, G, H, d, e, out.data_ptr(),
+          out.stride(0), _stream())
+
+
+def gated_delta_scan(tok: torch.Tensor, out: torch.Tensor, state: torch.Tensor, batch, kv_heads: int, heads: int,
+                     key_dim: int, value_dim: int) -> None:
+    """The gated delta rule, token by token through each sequence's state ``[slots, H, d, e]`` (float32):
+    ``S <- decay * S`` row by row; ``u = beta * (v - S^T k)``; ``S <- S + k u^T``; ``o = S^T q``. ``tok``: the rows of
+    ``delta_prepare``; ``out`` float32 ``[T, H e]``."""
+    G, H, d, e = kv_heads, heads, key_dim, value_dim
+    T = tok.shape[0]
+    _f32(tok, "delta rule rows", (T, 2 * G * d + H * e + H + H * d))
+    _f32(out, "delta rule output", (T, H * e))
+    _f32(state, "delta rule state")
+    if tuple(state.shape[1:]) != (H, d, e) or H % G or d > DELTA_RULE_MAX_DIM:
+        raise InvalidArgument(f"a state {list(state.shape)} does not fit {H} heads of {d} x {e} (keys up to "
+                              f"{DELTA_RULE_MAX_DIM}, {G} key heads)")
+    if batch.num_seqs == 0:
+        return
+    _call(_lib("delta_rule").tie_gated_delta_scan, "gated_delta_scan", tok.data_ptr(), tok.stride(0), out.data_ptr(),
+          out.stride(0), state.data_ptr(), batch.query_start.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs,
+          G, H, d, e, _stream())
+
+
+def grouped_gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor, out: torch.Tensor,
+                           groups: int) -> None:
+    """out = o / rms(o over each of ``groups`` equal groups of columns) * weight[column in its group] * sigmoid(gate).
+    ``o`` float32 ``[T, n]``, ``gate`` float32 rows of n (a view whose rows may lie further apart)."""
+    _f32(o, "gated norm input")
+    T, n = o.shape
+    if groups <= 0 or n % groups:
+        raise InvalidArgument(f"{n} columns are not {groups} equal groups")
+    _f32(weight, "gated norm weight", (n // groups,))
+    _gpu_strided(gate, "gate rows")
+    if gate.dtype != torch.float32 or tuple(gate.shape) != (T, n) or gate.stride(1) != 1:
+        raise InvalidArgument(f"gate rows {list(gate.shape)} {gate.dtype} do not fit float32 {[T, n]}")
+    _gpu(out, "gated norm output")
+    if tuple(out.shape) != (T, n):
+        raise InvalidArgument(f"gated norm output {list(out.shape)} does not match input {[T, n]}")
+    if T == 0:
+        return
+    _call(_lib("delta_rule").tie_grouped_gated_rms_norm, "grouped_gated_rms_norm", o.data_ptr(), o.stride(0),
+          weight.data_ptr(), float(eps), gate.data_ptr(), gate.stride(0), out.data_ptr(),
+          _code(out, "gated norm output"), T, groups, n // groups, _stream())
+
+
+# ------------------------------------------------- latent attention
+def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor, eps: float, angles: Optional[torch.Tensor],
+                   rotary_dim: int, pairing: str, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                   v_cache: Optional[torch.Tensor], block_size: int, write_kv: bool, q_plain: torch.Tensor,
+                   q_latent: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: int) -> None:
+    """Cache rows and query parts of a latent attention from the projection's float32 rows
+    ``[q: H x (dim + rot_dim) | latent (kv_rank) | rotated key part (rot_dim) | ...]``.
+
+    The latent is RMS-normed with ``latent_weight``; the key cache (one head of size D >= kv_rank + rot_dim) gets
+    ``[latent | rotated key part | zeros]``, the value cache ``[latent | zeros]``. ``q_plain`` ``[T, H dim]`` gets
+    the unrotated query parts, ``q_latent`` ``[T, H D]`` the rotated ones at columns ``kv_rank ..`` of every head
+    (zeros behind; columns below ``kv_rank`` are left for the product that takes the plain parts there)."""
+    _gpu_strided(proj, "projected rows")
+    T = proj.shape[0]
+    H, d, r, kr = heads, dim, rot_dim, kv_rank
+    D = q_latent.shape[1] // H
+    if proj.dtype != torch.float32 or proj.shape[1] < H * (d + r) + kr + r or proj.stride(1) != 1:
+        raise InvalidArgument(f"projected rows {list(proj.shape)} {proj.dtype} do not hold the queries and the latent")
+    _gpu(q_plain, "plain query parts")
+    _gpu(q_latent, "latent queries")
+    if tuple(q_plain.shape) != (T, H * d) or tuple(q_latent.shape) != (T, H * D) or D < kr + r or \
+            q_plain.dtype != q_latent.dtype:
+        raise InvalidArgument(f"query buffers {list(q_plain.shape)} / {list(q_latent.shape)} do not fit the heads")
+    _f32(latent_weight, "latent norm weight", (kr,))
+    if pairing not in ("rotate_half", "interleaved"):
+        raise InvalidArgument(f"pairs rotate as 'rotate_half' or 'interleaved', not '{pairing}'")
+    if rotary_dim:
+        _f32(angles, "rope angles", (T, rotary_dim))
+    cache_code = _code(q_plain, "queries")
+    if write_kv:
+        _i32(slots, "slot mapping", T)
+        _check_cache(k_cache, v_cache, 1, block_size, D)
+        cache_code = _cache_code(k_cache, q_plain, "k cache")
+    if T == 0:
+        return
+    _call(_lib("latent").tie_latent_prepare, "latent_prepare", proj.data_ptr(), proj.stride(0), latent_weight.data_ptr(),
+          float(eps), _ptr(angles) if rotary_dim else None, int(rotary_dim), int(pairing == "interleaved"),
+          _ptr(slots) if write_kv else None, _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
+          cache_code, block_size, int(write_kv), q_plain.data_ptr(), q_latent.data_ptr(), _code(q_plain, "queries"),
+          T, H, d, r, kr, D, _stream())
+
+
+def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
+    """``out[t, h] = w[h] @ x[t, h]`` for every head: ``x`` ``[T, H, K]``, ``w`` ``[H, N, K]``, ``out`` ``[T, H, N]``
+    (views whose rows and heads may lie further apart; the last dimension is dense), float32 sums; with ``gate``
+    (float32 ``[T, H, N]`` view) the result is multiplied by ``sigmoid(gate)``."""
+    for t, name in ((x, "head inputs"), (out, "head outputs")):
+        if not isinstance(t, torch.Tensor) or not t.is_cuda:
+            raise KernelUnavailable(f"{name} must be a tensor on a GPU: the engine's kernels have no CPU fallback")
+        if t.dim() != 3 or t.stride(2) != 1:
+            raise InvalidArgument(f"{name} {list(t.shape)} must be [rows, heads, width] with a dense last dimension")
+    _gpu(w, "head matrices")
+    T, H, K = x.shape
+    N = w.shape[1]
+    if tuple(w.shape) != (H, N, K) or tuple(out.shape) != (T, H, N):
+        raise InvalidArgument(f"head matrices {list(w.shape)} do not take {list(x.shape)} to {list(out.shape)}")
+    if gate is not None:
+        if not gate.is_cuda or gate.dim() != 3:
+            raise InvalidArgument("head gates must be a [rows, heads, width] tensor on the GPU")
+        if gate.dtype != torch.float32 or tuple(gate.shape) != (T, H, N) or gate.stride(2) != 1:
+            raise InvalidArgument(f"head gates {list(gate.shape)} {gate.dtype} do not fit float32 {[T, H, N]}")
+    if T == 0:
+        return
+    _call(_lib("latent").tie_head_linear, "head_linear", x.data_ptr(), _code(x, "head inputs"), x.stride(0), x.stride(1),
+          w.data_ptr(), _code(w, "head matrices"), out.data_ptr(), _code(out, "head outputs"), out.stride(0),
+          out.stride(1), _ptr(gate), gate.stride(0) if gate is not None else 0,
+          gate.stride(1) if gate is not None else 0, T, H, N, K, _stream())

@@ -196,7 +196,8 @@ class Model:
             _walk_parts(layer_parts, tensors, classes, set(), scalars)
             self._layer_tensors[index] = [(address, size) for address, size, _, _ in tensors]
             entry = self.cache_plan.calls[index]
-            binding = None if entry is None else (entry.group, entry.writes)
+            binding = None if entry is None else tuple((e.group, e.writes) for e in entry) \
+                if isinstance(entry, tuple) else (entry.group, entry.writes)
             ok = all(getattr(c, "replayable", False) for c in classes)
             names = {spec.name for part in layer_parts for spec in part.all_tensors()}
             signatures.append((tuple(classes), tuple(t[2:] for t in tensors), binding, _constants(scalars, names))
@@ -218,8 +219,12 @@ class Model:
                     end = start + 1
                     break
             # The same for the cache: entries that read an earlier entry's plane pass for "the same argument" too.
-            planes = {None if self.cache_plan.calls[i] is None else self.cache_plan.calls[i].plane
-                      for i in range(start, end)}
+            def plane_of(entry):
+                if entry is None:
+                    return None
+                return tuple(e.plane for e in entry) if isinstance(entry, tuple) else entry.plane
+
+            planes = {plane_of(self.cache_plan.calls[i]) for i in range(start, end)}
             if len(planes) not in (1, end - start):
                 end = start + 1
             if end - start >= self.MIN_ALIKE:
@@ -229,10 +234,11 @@ class Model:
     def _entry_tensors(self, ctx: StepContext, index: int, cache) -> list:
         """(address, bytes) of everything entry ``index`` owns on the device: its layer's tensors and its cache."""
         tensors = list(self._layer_tensors[index])
-        for name in ("k_cache", "v_cache", "state"):
-            t = getattr(cache, name, None)
-            if isinstance(t, torch.Tensor):
-                tensors.append((t.data_ptr(), t.numel() * t.element_size()))
+        for binding in (cache if isinstance(cache, tuple) else (cache,)):
+            for name in ("k_cache", "v_cache", "state"):
+                t = getattr(binding, name, None)
+                if isinstance(t, torch.Tensor):
+                    tensors.append((t.data_ptr(), t.numel() * t.element_size()))
         return tensors
 
     @staticmethod

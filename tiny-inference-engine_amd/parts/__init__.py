@@ -4,4 +4,5 @@ from .base import (Block, Embedding, FeedForward, Head, Mixer, Norm, PagedBindin
                    StateBinding,
                    StepContext, TensorSpec, Workspace, build_part, register_part, registered_parts,
                    unregister_part)
-from . import attention, block, embedding, feedforward, head, norm, position, recurrent  # noqa: F401  (registration)
+from . import (attention, block, embedding, feedforward, head, latent_attention, norm, parallel,  # noqa: F401
+               position, recurrent)  # noqa: F401  (registration)

@@ -38,6 +38,15 @@ Further parameters, for architectures that have them (absent or None: not applie
 * ``values_are_keys``: there is no value projection; the values are the keys as projected (with their bias), before
   the per-head norm and the rotation. ``names`` then has no ``v`` and ``bias`` none for it.
 
+* ``conv`` ``{"taps", "q", "k", "v"}`` (tensor names, each ``[channels, taps]``): a short causal convolution over time
+  on every channel of the projected q, k and v, directly behind the projection (before norm and rotation):
+  ``y_t = sum_j w[:, j] * u_(t - taps + 1 + j)``, zeros before the sequence's start. The last ``taps - 1`` projected
+  rows of a sequence are a state of fixed size, so the mixer then declares two needs (pages, state).
+* ``qk_norm`` with ``"over": "projection"``: q and k are RMS-normed over their whole projection at once (all heads
+  together, weights of that size) instead of head by head.
+* ``output_scale``: a factor on the mixer's result, folded into the convolution's value weights (float32) where there
+  is a convolution and into the output projection's weight otherwise.
+
 ``forward(..., residual=None)`` returns the mixer's output (float32 rows, or planes of partial sums) instead of
 adding it to a stream: for arrangements that norm a sub-layer's output first.
 """
@@ -49,7 +58,7 @@ from typing import List, Optional
 import torch
 
 from .. import kernels
-from ..cache.spec import PagedKV
+from ..cache.spec import FixedState, PagedKV
 from ..errors import InvalidArgument
 from .base import Mixer, Part, PartSpec, StepContext, TensorSpec, build_part, register_part
 from .linear import Linear
@@ -82,6 +91,14 @@ class PagedAttention(Mixer):
         self.stored_value_dim = int(params.get("value_dim") or self.head_dim)
         # Heads of unequal or odd size always; heads that nothing rotates or norms also where a size in steps of
         # 16 opens the matrix-core kernels.
+        self.qk_norm = params.get("qk_norm")
+        self.norm_over_projection = bool(self.qk_norm) and self.qk_norm.get("over") == "projection"
+        self.conv = dict(params["conv"]) if params.get("conv") else None
+        self.taps = int(self.conv["taps"]) if self.conv else 1
+        if self.conv and not 1 <= self.taps <= kernels.CONV_MAX_TAPS:
+            raise InvalidArgument(f"a convolution of {self.taps} taps: 1 to {kernels.CONV_MAX_TAPS} are supported")
+        self.output_scale = float(params.get("output_scale", 1.0))
+        self.conv_weight: torch.Tensor = None
         plain_heads = not params.get("qk_norm") and (params.get("position") or PartSpec("none")).kind == "none" \
             and not params.get("bias")
         self.padded = self.stored_value_dim != self.stored_key_dim or self.head_dim % 2 != 0 or \
@@ -102,6 +119,9 @@ class PagedAttention(Mixer):
             raise InvalidArgument("the q, k and v projections run as one product: a bias for all of them or for none")
         if self.padded and bias:
             raise InvalidArgument("heads padded to a common size take no bias")
+        if (self.conv or self.norm_over_projection) and (self.values_are_keys or bias or self.value_mix is not None):
+            raise InvalidArgument("a convolution or a norm over the whole projection goes with plain q, k and v "
+                                  "projections: no bias, no blended values, no values that are the keys")
         if self.values_are_keys and (self.padded or self.value_mix is not None or "v" in names or "v" in bias):
             raise InvalidArgument("values that are the keys have the keys' size, no projection of their own and no blend")
         stored = [self.num_heads * self.stored_key_dim, self.num_kv_heads * self.stored_key_dim,
@@ -118,7 +138,6 @@ class PagedAttention(Mixer):
                           bias=[bias[k] for k in inputs] if "q" in bias and not self.bias_in_kernel else None)
         self.out = Linear([names["o"]], [self.hidden], self.num_heads * self.stored_value_dim if self.padded else q_dim,
                           bias=[bias["o"]] if "o" in bias else None)
-        self.qk_norm = params.get("qk_norm")
         self.q_norm_weight: torch.Tensor = None
         self.k_norm_weight: torch.Tensor = None
         position: PartSpec = params.get("position") or PartSpec("none")
@@ -126,14 +145,22 @@ class PagedAttention(Mixer):
         if self.values_are_keys and self.position.rotary_table() is None:
             raise InvalidArgument("values that are the keys need a position encoding the fused kernel applies: any "
                                   "other changes the projected keys in place before they are cached as values")
-        if self.padded and (self.qk_norm or position.kind != "none"):
-            raise InvalidArgument("heads whose key and value sizes differ take no per-head norm and no rotation")
+        table = self.position.rotary_table()
+        rotates_only = table is not None and (table[0] is not None or not table[1]) and \
+            int(table[1] or 0) <= self.stored_key_dim
+        if self.padded and ((self.qk_norm and not self.norm_over_projection) or
+                            (position.kind != "none" and not rotates_only)):
+            raise InvalidArgument("heads whose key and value sizes differ take no per-head norm, and a rotation only "
+                                  "of dimensions the stored keys have")
 
     def children(self) -> List[Part]:
         return [self.position]
 
     def cache_need(self):
-        return PagedKV(self.num_kv_heads, self.head_dim, self.window, self.chunk)
+        pages = PagedKV(self.num_kv_heads, self.head_dim, self.window, self.chunk)
+        if self.taps > 1:
+            return (pages, FixedState((self.taps - 1, self.q_dim + 2 * self.kv_dim)))
+        return pages
 
     def tensors(self) -> List[TensorSpec]:
         specs = self.qkv.tensors() + self.out.tensors()
@@ -142,8 +169,15 @@ class PagedAttention(Mixer):
                       for b, o in zip(self.qkv_bias_names, self.qkv.out_features)]
         if self.qk_norm:
             init = ("one_plus_uniform", 0.1)
-            specs.append(TensorSpec(self.qk_norm["q_weight"], (self.head_dim,), "vector", init))
-            specs.append(TensorSpec(self.qk_norm["k_weight"], (self.head_dim,), "vector", init))
+            sizes = (self.num_heads * self.stored_key_dim, self.num_kv_heads * self.stored_key_dim) \
+                if self.norm_over_projection else (self.head_dim, self.head_dim)
+            specs.append(TensorSpec(self.qk_norm["q_weight"], (sizes[0],), "vector", init))
+            specs.append(TensorSpec(self.qk_norm["k_weight"], (sizes[1],), "vector", init))
+        if self.conv:
+            for key, heads, width in (("q", self.num_heads, self.stored_key_dim),
+                                      ("k", self.num_kv_heads, self.stored_key_dim),
+                                      ("v", self.num_kv_heads, self.stored_value_dim)):
+                specs.append(TensorSpec(self.conv[key], (heads * width, self.taps), "vector", ("normal", 0.4)))
         if self.value_mix is not None and self.value_mix.get("weight"):
             specs.append(TensorSpec(self.value_mix["weight"], (1,), "vector", ("normal", 0.3)))   # a stored scalar reads as [1]
         if self.sink_name:
@@ -167,18 +201,41 @@ class PagedAttention(Mixer):
         o[:, :, :self.stored_value_dim] = w.view(self.hidden, self.num_heads, self.stored_value_dim)
         self.out.set_weight(o.view(self.hidden, self.q_dim).contiguous())
 
+    def _per_channel(self, t: torch.Tensor, heads: int, stored: int) -> torch.Tensor:
+        """A stored per-channel tensor ``[heads * stored, ...]`` at the heads' common size (zeros for what a head lacks)."""
+        t = t.to(torch.float32).reshape(heads, stored, -1)
+        if stored != self.head_dim:
+            wide = t.new_zeros((heads, self.head_dim, t.shape[2]))
+            wide[:, :stored] = t
+            t = wide
+        return t.reshape(heads * self.head_dim, -1)
+
     def load(self, fetch, mode, device) -> None:
         if self.padded:
             self._load_padded(fetch)
         else:
             self.qkv.load(fetch)
             self.out.load(fetch)
+        H, KVH = self.num_heads, self.num_kv_heads
+        if self.conv:
+            parts = [self._per_channel(fetch(self.conv["q"], "vector"), H, self.stored_key_dim),
+                     self._per_channel(fetch(self.conv["k"], "vector"), KVH, self.stored_key_dim),
+                     self._per_channel(fetch(self.conv["v"], "vector"), KVH, self.stored_value_dim) * self.output_scale]
+            self.conv_weight = torch.cat(parts).contiguous()
+        elif self.output_scale != 1.0:
+            w = self.out.weight
+            if isinstance(w, kernels.PackedWeight):
+                raise InvalidArgument("an output scale without a convolution must be folded before the weight is packed")
+            self.out.set_weight((w.to(torch.float32) * self.output_scale).to(w.dtype))
         if self.value_mix is not None and self.value_mix.get("weight"):
             weight = fetch(self.value_mix["weight"], "vector")
             self.value_mix_weight = weight.reshape(1).contiguous() if self.value_mix["role"] == "blend" else None
         if self.qk_norm:
             self.q_norm_weight = fetch(self.qk_norm["q_weight"], "vector")
             self.k_norm_weight = fetch(self.qk_norm["k_weight"], "vector")
+            if self.norm_over_projection:
+                self.q_norm_weight = self._per_channel(self.q_norm_weight, H, self.stored_key_dim).reshape(-1).contiguous()
+                self.k_norm_weight = self._per_channel(self.k_norm_weight, KVH, self.stored_key_dim).reshape(-1).contiguous()
         if self.sink_name:
             self.sinks = fetch(self.sink_name, "vector").to(torch.float32).contiguous()
         if self.qkv_bias_names is not None:
@@ -196,6 +253,12 @@ class PagedAttention(Mixer):
         result = ctx.scratch("attention.result", (attn.shape[0], self.hidden), torch.float32)
         self.out(attn, result, accumulate=False, ctx=ctx)
         return result
+
+    def _unit_conv(self, device) -> torch.Tensor:
+        """The weights of a convolution of one tap that changes nothing (a norm over the projection without one)."""
+        if self.conv_weight is None:
+            self.conv_weight = torch.ones((self.q_dim + 2 * self.kv_dim, 1), dtype=torch.float32, device=device)
+        return self.conv_weight
 
     def _kernel_bias(self, writes: bool) -> Optional[torch.Tensor]:
         """The bias as the cache-write kernel takes it: of the columns it reads (q alone where it writes no keys)."""
@@ -215,22 +278,40 @@ class PagedAttention(Mixer):
     def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: Optional[torch.Tensor]):
         T = h.shape[0]
         H, KVH, Dh = self.num_heads, self.num_kv_heads, self.head_dim
+        conv_state = None
+        if isinstance(cache, tuple):          # pages, and the convolution's last inputs
+            cache, conv_state = cache[0], cache[1].state
         step = cache.step
         eps = float(self.qk_norm["eps"]) if self.qk_norm else 0.0
+        q_weight, k_weight = (self.q_norm_weight, self.k_norm_weight) if self.qk_norm else (None, None)
 
         width = self.q_dim + (1 if self.values_are_keys else 2) * self.kv_dim
         q = ctx.scratch("attention.q", (T, self.q_dim))
         table = self.position.rotary_table()
         # Decode-size steps: the projection comes as planes of partial sums, added by the kernel that reads them.
-        planes = self.qkv.partial_planes(ctx, h, "attention.qkv") if table is not None else None
+        rows_first = self.conv is not None or self.norm_over_projection
+        planes = self.qkv.partial_planes(ctx, h, "attention.qkv") if table is not None and not rows_first else None
         if planes is not None:
             qkv = planes[0]
         else:
             qkv = ctx.scratch("attention.qkv", (T, width), torch.float32)
             self.qkv(h, qkv, ctx=ctx)
+        if rows_first:
+            # The convolution over time (from the rows as projected and the sequence's state) and the norms over a
+            # whole projection, one kernel; the kernels below then neither norm nor see the raw rows.
+            raw, qkv = qkv, ctx.scratch("attention.qkv_conv", (T, width), torch.float32)
+            kernels.conv_qkv(raw, self.conv_weight if self.conv else self._unit_conv(raw.device), self.taps, conv_state,
+                             ctx.batch, (self.q_dim, self.kv_dim, self.kv_dim), qkv,
+                             q_weight if self.norm_over_projection else None,
+                             k_weight if self.norm_over_projection else None,
+                             (H * self.stored_key_dim, KVH * self.stored_key_dim), eps)
+            if conv_state is not None and cache.writes:
+                kernels.conv_state_update(raw, self.taps, conv_state, ctx.batch, width)
+            if self.norm_over_projection:
+                q_weight = k_weight = None
         if table is not None:
             inv_freq, rotary_dim, pairing = table
-            if (inv_freq is not None and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
+            if (inv_freq is not None and not rows_first and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
                     and self.value_mix is None and not self.values_are_keys and not self.chunk and self.sinks is None
                     and self.qkv_bias is None
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
@@ -239,13 +320,13 @@ class PagedAttention(Mixer):
                 attn = ctx.scratch("attention.out", (T, self.q_dim))
                 kernels.paged_attention_prepared(
                     planes if planes is not None else qkv.unsqueeze(0),
-                    self.q_norm_weight if self.qk_norm else None, self.k_norm_weight if self.qk_norm else None, eps, self.position.angles(ctx), cache.writes, cache.k_cache, cache.v_cache, attn, step, ctx.batch,
+                    q_weight, k_weight, eps, self.position.angles(ctx), cache.writes, cache.k_cache, cache.v_cache, attn, step, ctx.batch,
                     H, self.scale, self.window, ctx.scratch)
                 return self._finish(ctx, attn, residual)
             if inv_freq is None:                      # an encoding that leaves queries and keys as they are
                 rotary_dim, pairing = None, "rotate_half"
             kernels.qk_norm_rope_kv_write(
-                qkv, q, self.q_norm_weight, self.k_norm_weight, eps, inv_freq, ctx.batch.positions,
+                qkv, q, q_weight, k_weight, eps, inv_freq, ctx.batch.positions,
                 step.slot_mapping, cache.k_cache, cache.v_cache, H, KVH, Dh, cache.block_size,
                 write_kv=cache.writes, planes=1 if planes is None else planes.shape[0], plane_stride=T * width,
                 angles=self.position.angles(ctx) if inv_freq is not None else None,
@@ -256,9 +337,9 @@ class PagedAttention(Mixer):
             # change q and k (float32 views into the projection rows), then convert and store.
             q_view = qkv[:, :self.q_dim]
             k_view = qkv[:, self.q_dim:self.q_dim + self.kv_dim]
-            if self.qk_norm:
+            if q_weight is not None:
                 kernels.qk_norm_rope_kv_write(
-                    qkv, q_view, self.q_norm_weight, self.k_norm_weight, eps, None, ctx.batch.positions,
+                    qkv, q_view, q_weight, k_weight, eps, None, ctx.batch.positions,
                     None, None, None, H, KVH, Dh, cache.block_size, write_kv=False, k_dense=k_view)
             self.position.apply(ctx, q_view.unflatten(1, (H, Dh)), k_view.unflatten(1, (KVH, Dh)),
                                 ctx.batch.positions)

@@ -250,11 +250,16 @@ class StepContext:
 
     def cache_of(self, call_index: int):
         """The cache binding of run-order entry ``call_index`` (None if its mixer has no cache)."""
-        from ..cache.spec import PagedKV
-
         entry = self.cache_plan.calls[call_index]
         if entry is None:
             return None
+        if isinstance(entry, tuple):         # a mixer that declared several needs: one binding a need, in its order
+            return tuple(self._bind(e) for e in entry)
+        return self._bind(entry)
+
+    def _bind(self, entry):
+        from ..cache.spec import PagedKV
+
         need = self.cache_plan.groups[entry.group].need
         if isinstance(need, PagedKV):
             k, v = self.cache_manager.kv_planes(entry.group, entry.plane)
@@ -325,7 +330,8 @@ class Position(Part):
 
 class Mixer(Part):
     def cache_need(self):
-        """What this mixer needs from the cache: a PagedKV, a FixedState, or None."""
+        """What this mixer needs from the cache: a PagedKV, a FixedState, None, or a tuple of several of them
+        (``forward`` then receives a tuple of bindings in the same order)."""
         return None
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache, residual: torch.Tensor) -> None:

@@ -10,14 +10,26 @@ half alone (and needs that half's norm only).
 ``x += post_feed_forward(feed_forward(pre_feed_forward(x)))``. The sub-layers are asked for their result instead of
 adding it (``forward(..., residual=None)``); the norm over the result, the addition to the stream and the norm
 that the stream meets next run as one kernel where the norms can (``Norm.add_normed``).
+
+``hyper_connections`` keeps ``streams`` copies of the residual instead of one. All start as the embedding's rows.
+Sub-layer q of a layer (its mixer, then its feed-forward) has three small tensors ``in`` ``[streams]``, ``out``
+``[streams]`` and ``mix`` ``[streams, streams]`` (from, to): it reads ``u = sum_s in[s] x_s``, computes
+``y = sublayer(norm(u))``, and every stream becomes ``x_t <- sum_s mix[s, t] x_s + out[t] y``, all from the old
+streams. The model's single residual row receives the sum of the streams behind every layer (what the head
+norms, and what a layer hook sees). The streams live in step scratch memory: they never outlast a step. One
+kernel does a sub-layer's write and the next sub-layer's read with its norm. Parameters: ``streams``, ``hidden``,
+``names`` (``mixer`` and ``feed_forward``, each ``{"in", "out", "mix"}``).
 """
 
 from __future__ import annotations
 
+from typing import List
+
 import torch
 
+from .. import kernels
 from ..errors import InvalidArgument
-from .base import Block, StepContext, register_part
+from .base import Block, StepContext, TensorSpec, register_part
 
 
 @register_part("block", "pre_norm")
@@ -97,3 +109,97 @@ class SandwichNormBlock(Block):
         missing = [n for n in needed if n not in layer.norms]
         if missing:
             raise InvalidArgument(f"a sandwich_norm block needs the norms {', '.join(needed)}; missing {', '.join(missing)}")
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionsBlock(Block):
+    capturable = True
+    replayable = False     # the first block of a step makes the streams: what a layer launches depends on its place
+    NORMS = ("pre_mixer", "pre_feed_forward")
+    SUBLAYERS = ("mixer", "feed_forward")
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.streams = int(params["streams"])
+        self.hidden = int(params["hidden"])
+        if not 0 < self.streams <= kernels.HYPER_MAX_STREAMS:
+            raise InvalidArgument(f"{self.streams} residual streams: 1 to {kernels.HYPER_MAX_STREAMS} are supported")
+        self.names = {k: dict(v) for k, v in params["names"].items()}
+        self.weights = {}
+
+    def tensors(self) -> List[TensorSpec]:
+        s, specs = self.streams, []
+        for names in self.names.values():
+            specs.append(TensorSpec(names["in"], (s,), "vector", ("normal", 0.5)))
+            specs.append(TensorSpec(names["out"], (s,), "vector", ("one_plus_uniform", 0.2)))
+            specs.append(TensorSpec(names["mix"], (s, s), "vector", ("normal", 0.4)))
+        return specs
+
+    def load(self, fetch, mode, device) -> None:
+        for sub, names in self.names.items():
+            self.weights[sub] = tuple(fetch(names[k], "vector").to(torch.float32).contiguous()
+                                      for k in ("in", "out", "mix"))
+
+    @classmethod
+    def check_layer(cls, layer) -> None:
+        needed = [n for n, part in zip(cls.NORMS, (layer.mixer, layer.feed_forward)) if part is not None]
+        if not needed:
+            raise InvalidArgument("a hyper_connections block needs a mixer, a feed-forward or both")
+        missing = [n for n in needed if n not in layer.norms]
+        missing += [s for s, part in zip(cls.SUBLAYERS, (layer.mixer, layer.feed_forward))
+                    if part is not None and s not in layer.block.names]
+        if missing:
+            raise InvalidArgument(f"a hyper_connections block lacks {', '.join(missing)}")
+
+    def _read(self, ctx: StepContext, sub: str, norm, T: int):
+        """What the pass over the streams needs to also make the rows sub-layer ``sub`` reads: the kernel applies a
+        layer norm or an RMS norm itself and hands any other norm the float32 sum."""
+        kind = {"LayerNorm": "layer_norm", "RMSNorm": "rms_norm"}.get(type(norm).__name__)
+        if kind is not None and hasattr(norm, "weight") and hasattr(norm, "eps"):
+            h = ctx.scratch("hyper.normed", (T, self.hidden), ctx.act_dtype)
+            ctx.set_row_scale(h, None)
+            return (self.weights[sub][0], kind, norm.weight, norm.eps, h), h, None
+        u = ctx.scratch("hyper.sum", (T, self.hidden), torch.float32)
+        return (self.weights[sub][0], None, None, 0.0, u), None, u
+
+    @staticmethod
+    def _result(ctx: StepContext, part, run, T: int, hidden: int) -> torch.Tensor:
+        """The sub-layer's result as float32 rows or planes of partial sums."""
+        if getattr(part, "returns_result", False):
+            y = run(None)
+            ctx.settle()
+            if isinstance(y, torch.Tensor):
+                return y
+            rows = ctx.scratch("hyper.sublayer_result", (T, hidden), torch.float32)
+            kernels.moe_combine(y, rows)            # a routed feed-forward's parts
+            return rows
+        zeros = ctx.scratch("hyper.sublayer_result", (T, hidden), torch.float32)
+        zeros.zero_()
+        run(zeros)
+        ctx.settle()
+        return zeros
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
+        T = x.shape[0]
+        ctx.settle()
+        streams = ctx.scratch("hyper.streams", (self.streams, T, self.hidden), torch.float32)
+        subs = [(s, part, layer.norms[n]) for s, n, part in
+                zip(self.SUBLAYERS, self.NORMS, (layer.mixer, layer.feed_forward)) if part is not None]
+        fresh = ctx.notes.get("hyper.streams") is None     # the first layer of the step: the streams are x
+        ctx.notes["hyper.streams"] = streams
+        read, h, u = self._read(ctx, subs[0][0], subs[0][2], T)
+        kernels.hyper_connection(streams, x, from_x=fresh, read=read)
+        for i, (sub, part, norm) in enumerate(subs):
+            if h is None:
+                h = norm.forward(ctx, u)
+            rows = h
+            if sub == "mixer":
+                y = self._result(ctx, part, lambda residual: part.forward(ctx, rows, cache, residual), T, self.hidden)
+            else:
+                y = self._result(ctx, part, lambda residual: part.forward(ctx, rows, residual), T, self.hidden)
+            last = i + 1 == len(subs)
+            read = h = u = None
+            if not last:
+                read, h, u = self._read(ctx, subs[i + 1][0], subs[i + 1][2], T)
+            _, out_w, mix = self.weights[sub]
+            kernels.hyper_connection(streams, x, fold=last, write=(y, mix, out_w), read=read)

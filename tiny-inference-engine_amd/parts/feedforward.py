@@ -7,7 +7,9 @@ to right, ``out = a @ Wd^T``, added to the residual; no bias, no experts
 (``src/model/qwen3.cpp:235-239``, ``src/backend/cpu/cpu_backend.cpp:195-207``).
 Gate and up run as one product over the two matrices side by side; with bfloat16 weights
 their rows are interleaved in blocks of 8 and the product's epilogue applies the activation.
-Parameters: ``hidden``, ``intermediate``, ``names`` (``gate``, ``up``, ``down``).
+Parameters: ``hidden``, ``intermediate``, ``names`` (``gate``, ``up``, ``down``) and, for designs whose gate goes
+through another function, ``activation``: ``silu`` (the default) or ``gelu_tanh``,
+``0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))``.
 
 ``mlp`` is ``down(act(up(h)))`` without a gate; ``activation`` names the function (``gelu``: the exact form,
 ``0.5 z (1 + erf(z / sqrt 2))``; ``poly_norm``: ``a N(z) + b N(z^2) + c N(z^3) + e`` with powers taken element by
@@ -56,6 +58,10 @@ class SwiGLU(FeedForward):
         super().__init__(params)
         self.hidden = int(params["hidden"])
         self.intermediate = int(params["intermediate"])
+        self.activation = params.get("activation") or "silu"
+        if self.activation not in kernels.GATE_ACTIVATIONS:
+            raise UnsupportedError(f"a gate's activation '{self.activation}' (supported: "
+                                   f"{', '.join(kernels.GATE_ACTIVATIONS)})")
         names = params["names"]
         self.gate_up = Linear([names["gate"], names["up"]], [self.intermediate, self.intermediate], self.hidden)
         self.down = Linear([names["down"]], [self.hidden], self.intermediate)
@@ -79,11 +85,12 @@ class SwiGLU(FeedForward):
         T = h.shape[0]
         act = ctx.scratch("swiglu.act", (T, self.intermediate))
         if self.fused and h.dtype == torch.bfloat16:
-            kernels.linear_swiglu(h, self.gate_up.weight, act, row_scale=Linear.row_scale_for(ctx, h, self.gate_up.weight))
+            kernels.linear_swiglu(h, self.gate_up.weight, act, row_scale=Linear.row_scale_for(ctx, h, self.gate_up.weight),
+                                  activation=self.activation)
         else:
             gate_up = ctx.scratch("swiglu.gate_up", (T, 2 * self.intermediate))
             self.gate_up(h, gate_up, ctx=ctx)
-            kernels.swiglu(gate_up, act)
+            kernels.swiglu(gate_up, act, self.activation)
         return _finish(ctx, self.down, act, residual, "feed_forward.result")
 
 

@@ -1,4 +1,4 @@
-"""RMSNorm: ``out = (x * inv) * w`` with ``inv = 1 / sqrt(mean(x^2) + eps)``.
+"""Norms over the rows of the stream. RMSNorm: ``out = (x * inv) * w`` with ``inv = 1 / sqrt(mean(x^2) + eps)``.
 
 The weight multiplies after normalisation and is the plain ``w`` (not ``1 + w``);
 no bias, no mean subtraction; statistics in float32
@@ -6,6 +6,9 @@ no bias, no mean subtraction; statistics in float32
 ``weight`` (tensor name) and, for designs that store the weight around zero, ``one_plus`` (True: the norm
 multiplies by ``1 + w``; the sum is formed once at load time, in float32, which is the value the multiplication
 would see anyway).
+
+``layer_norm`` subtracts the row's mean first: ``out = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w``, a weight and
+no bias, statistics in float32. Parameters: ``dim``, ``eps``, ``weight``.
 
 ``add_normed`` is the norm applied to a sub-layer's OUTPUT on its way into the stream, for arrangements that norm
 both sides of a sub-layer: ``x += RMSNorm(y) * w``, optionally with the next norm of the stream in the same pass.
@@ -83,4 +86,31 @@ class RMSNorm(Norm):
             ctx.set_row_scale(out, None)
         kernels.norm_add_norm(y, self.weight, self.eps, x, next_norm.weight if next_norm is not None else None,
                               next_norm.eps if next_norm is not None else 0.0, out)
+        return out
+
+
+@register_part("norm", "layer_norm")
+class LayerNorm(Norm):
+    capturable = True
+    replayable = True
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.dim = int(params["dim"])
+        self.eps = float(params["eps"])
+        self.weight_name = params["weight"]
+        self.weight: torch.Tensor = None
+
+    def tensors(self) -> List[TensorSpec]:
+        return [TensorSpec(self.weight_name, (self.dim,), "vector", ("one_plus_uniform", 0.1))]
+
+    def load(self, fetch, mode, device) -> None:
+        self.weight = fetch(self.weight_name, "vector")
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
+        count = x.shape[0] if rows is None else rows.numel()
+        out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
+        ctx.set_row_scale(out, None)
+        kernels.layer_norm(x, self.weight, self.eps, out, rows)
         return out

@@ -9,9 +9,21 @@ and keys are, values are not. Parameters: ``head_dim``, ``theta``.
 For designs that have them: ``rotary_dim`` r (even, at most ``head_dim``): only the first r dimensions of a head
 rotate, dimension i paired with i + r/2 and ``inv_freq[i] = theta^(-2i / r)``, the others pass unchanged;
 ``scaling_factor`` f (linear position scaling): every frequency is divided by f.
+
+``rope_yarn`` is a rotation whose frequencies are stretched for contexts longer than the one they were made for
+(YaRN): with ``f_i = theta^(-2i / r)`` over the r rotated dimensions and ``scaling`` = (factor, original, fast, slow),
+
+    dim(t) = r ln(original / (2 pi t)) / (2 ln theta),  lo = max(floor(dim(fast)), 0),  hi = min(ceil(dim(slow)), r - 1),
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),   frequency_i = f_i / factor * ramp_i + f_i (1 - ramp_i),
+
+and both the cosine and the sine are multiplied by ``0.1 ln(factor) + 1``. Without ``scaling`` it is the plain
+rotation. ``pairing`` says which dimensions form a pair: ``rotate_half`` (i, i + r/2) or ``interleaved`` (2i, 2i + 1).
+Parameters: ``head_dim``, ``theta``, ``rotary_dim``, ``pairing``, ``scaling``.
 """
 
 from __future__ import annotations
+
+import math
 
 import numpy as np
 import torch
@@ -77,3 +89,64 @@ class NoPosition(Position):
 
     def rotary_table(self):
         return None, 0, "none"
+
+
+@register_part("position", "rope_yarn")
+class RopeYarn(Position):
+    capturable = True
+    replayable = True
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.head_dim = int(params["head_dim"])
+        self.theta = float(params["theta"])
+        self.rotary_dim = int(params.get("rotary_dim") or self.head_dim)
+        self.pairing = params.get("pairing", "rotate_half")
+        self.scaling = dict(params["scaling"]) if params.get("scaling") else None
+        if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
+            raise InvalidArgument(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
+        if self.pairing not in ("rotate_half", "interleaved"):
+            raise InvalidArgument(f"pairs rotate as 'rotate_half' or 'interleaved', not '{self.pairing}'")
+        if not self.theta > 0 or self.theta == 1.0:
+            raise InvalidArgument(f"rope theta must be positive and not 1, got {self.theta}")
+        self.amplitude = 1.0
+        if self.scaling is not None:
+            for key in ("factor", "original", "fast", "slow"):
+                if not float(self.scaling[key]) > 0:
+                    raise InvalidArgument(f"rope scaling {key} must be positive, got {self.scaling[key]}")
+            self.amplitude = 0.1 * math.log(float(self.scaling["factor"])) + 1.0
+        self.inv_freq: torch.Tensor = None
+
+    def host_inv_freq(self) -> np.ndarray:
+        """The frequencies in double precision, rounded to float32 once."""
+        r = self.rotary_dim
+        i = np.arange(r // 2, dtype=np.float64)
+        freq = np.power(self.theta, -2.0 * i / r)
+        if self.scaling is not None:
+            factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+
+            def dim_of(turns: float) -> float:
+                return r * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+            lo = max(math.floor(dim_of(float(self.scaling["fast"]))), 0)
+            hi = min(math.ceil(dim_of(float(self.scaling["slow"]))), r - 1)
+            ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            freq = freq / factor * ramp + freq * (1.0 - ramp)
+        return freq.astype(np.float32)
+
+    def load(self, fetch, mode, device) -> None:
+        self.inv_freq = torch.from_numpy(self.host_inv_freq()).to(device)
+
+    def rotary_table(self):
+        return self.inv_freq, self.rotary_dim, self.pairing
+
+    def angles(self, ctx) -> torch.Tensor:
+        """amplitude * (cos | sin) of this step's positions, ``[T, rotary_dim]`` float32: once a step for all layers
+        with the same frequencies."""
+        key = ("rope_yarn", self.rotary_dim, self.theta, repr(sorted((self.scaling or {}).items())))
+        table = ctx.notes.get(key)
+        if table is None:
+            table = ctx.scratch("rope.angles:" + repr(key), (ctx.num_tokens, self.rotary_dim), torch.float32)
+            kernels.rope_angles(ctx.batch.positions, self.inv_freq, table, self.amplitude)
+            ctx.notes[key] = table
+        return table

@@ -48,6 +48,20 @@ class TensorSpec:
     role: str = "matrix"                     # "matrix", "vector" or "int_table"
     init: Tuple = ("normal", 0.02)           # how random-weights mode fills it
     optional: bool = False                   # may be absent; if present it is shape-checked
+    # A dimension given as None is whatever the file holds (an inner size no configuration key names);
+    # ``free_dims`` lists, in order, the sizes random-weights mode gives such dimensions.
+    free_dims: Tuple[int, ...] = ()
+
+    def concrete_shape(self) -> Tuple[int, ...]:
+        free = list(self.free_dims)
+        try:
+            return tuple(d if d is not None else free.pop(0) for d in self.shape)
+        except IndexError:
+            raise InvalidArgument(f"tensor '{self.name}' has a free dimension and no size to make it with") from None
+
+    def fits(self, shape) -> bool:
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(d is None or d == got for d, got in zip(self.shape, shape))
 
 
 def check_tensors(expected: Iterable[TensorSpec], stored: Dict[str, StoredTensor], what: str = "the model") -> None:
@@ -65,8 +79,9 @@ def check_tensors(expected: Iterable[TensorSpec], stored: Dict[str, StoredTensor
             if not spec.optional:
                 missing.append(spec.name)
             continue
-        if tuple(tensor.shape) != tuple(spec.shape):
-            wrong_shape.append(f"{spec.name}: has {list(tensor.shape)}, expected {list(spec.shape)}")
+        if not spec.fits(tensor.shape):
+            wrong_shape.append(f"{spec.name}: has {list(tensor.shape)}, expected "
+                               f"{['any' if d is None else d for d in spec.shape]}")
         allowed = _INT if spec.role == "int_table" else _FLOAT
         if tensor.dtype not in allowed:
             wrong_dtype.append(f"{spec.name}: has {tensor.dtype}, expected one of {', '.join(allowed)}")

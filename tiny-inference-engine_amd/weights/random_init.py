@@ -128,20 +128,20 @@ def random_tensor(spec: TensorSpec, seed: int, dtype: torch.dtype, device="cpu")
     bits on the host and on a GPU."""
     kind = spec.init[0]
     if spec.role == "int_table":
-        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
+        return torch.zeros(spec.concrete_shape(), dtype=torch.int32, device=device)
     if kind == "zeros":
-        return torch.zeros(spec.shape, dtype=dtype, device=device)
+        return torch.zeros(spec.concrete_shape(), dtype=dtype, device=device)
     if kind not in ("normal", "one_plus_uniform"):
         raise InvalidArgument(f"tensor '{spec.name}' has unknown init '{kind}'")
     key, scale = _stream_seed(seed, spec.name), float(spec.init[1])
     count = 1
-    for d in spec.shape:
+    for d in spec.concrete_shape():
         count *= int(d)
     if torch.device(device).type == "cpu":
-        return _draw_on_host(key, count, kind, scale).reshape(tuple(spec.shape)).to(dtype)
+        return _draw_on_host(key, count, kind, scale).reshape(spec.concrete_shape()).to(dtype)
     from .. import kernels
 
-    t = torch.empty(spec.shape, dtype=torch.float32, device=device)
+    t = torch.empty(spec.concrete_shape(), dtype=torch.float32, device=device)
     kernels.random_fill(t, key, kind, scale)
     return t.to(dtype)
 
@@ -173,7 +173,7 @@ def write_random_model(folder, config_values: dict, seed: int, dtype: str = "bfl
         if s.name in seen:
             continue
         seen.add(s.name)
-        declared.append((s.name, tuple(s.shape), torch.int32 if s.role == "int_table" else store))
+        declared.append((s.name, s.concrete_shape(), torch.int32 if s.role == "int_table" else store))
     write_safetensors(folder / "model.safetensors", random_tensors(specs, seed, store, device),
                       shapes_and_dtypes=declared, metadata={"format": "pt", "seed": seed})
     return str(folder)
