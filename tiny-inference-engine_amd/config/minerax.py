@@ -11,7 +11,8 @@ feed-forward (or none). Nothing about a layer is assumed from another layer. Key
     max_positions         optional: the longest sequence (default 131072; the design itself has no limit)
     layers[i].type        "latent_attention" or "parallel"
     layers[i].mixer       latent_attention: heads, dim, rot_dim, vdim, kv_rank, scale, mask.size (optional: a sliding
-                                            window), rot.{dims, base, scaling.{factor, original, fast, slow}}
+                                            window), rot.{dims, base, scaling.{factor, original, fast, slow}} (optional,
+                                            as is its scaling)
                           parallel: left_scale, right_scale,
                                     left.{heads, kv_heads, dim, vdim, conv, scale, softcap (optional), rot (as above,
                                           optional), mask.size (optional)},
@@ -53,7 +54,7 @@ class LatentAttentionConfig:
     kv_rank: int                  # size of the cached latent
     scale: float
     window: Optional[int]
-    rotation: RotationConfig
+    rotation: Optional[RotationConfig]
 
 
 @dataclasses.dataclass(frozen=True)
@@ -143,7 +144,7 @@ class MineraxConfig:
         heads, dim, rot_dim = r.integer("heads"), r.integer("dim"), r.integer("rot_dim")
         vdim, kv_rank, scale = r.integer("vdim", dim), r.integer("kv_rank"), r.number("scale")
         _positive(where, heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=scale)
-        rotation = _rotation(_section(r, "rot", where), where, rot_dim)
+        rotation = _rotation(_section(r, "rot", where, required=False), where, rot_dim)
         return LatentAttentionConfig(heads, dim, rot_dim, vdim, kv_rank, scale, _window(r, where), rotation)
 
     @staticmethod

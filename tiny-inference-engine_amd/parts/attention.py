@@ -146,8 +146,7 @@ class PagedAttention(Mixer):
             raise InvalidArgument("values that are the keys need a position encoding the fused kernel applies: any "
                                   "other changes the projected keys in place before they are cached as values")
         table = self.position.rotary_table()
-        rotates_only = table is not None and (table[0] is not None or not table[1]) and \
-            int(table[1] or 0) <= self.stored_key_dim
+        rotates_only = table is not None and int(table[1] or 0) <= self.stored_key_dim
         if self.padded and ((self.qk_norm and not self.norm_over_projection) or
                             (position.kind != "none" and not rotates_only)):
             raise InvalidArgument("heads whose key and value sizes differ take no per-head norm, and a rotation only "
