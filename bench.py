@@ -109,10 +109,50 @@ def qwen3_beside_topapel(size):
                 intermediate_size=size["ff"] * 2 // 3, vocab_size=size["vocab"])
 
 
+# ``--workload minerax``: the Minerax design at sizes that resemble a real model's layers, beside Qwen3 with the same
+# stream, as many heads of the same size and a gated feed-forward as wide. Layers repeat (three with latent attention
+# over a sliding window, one with convolved attention beside a gated delta rule); two residual streams. The cached
+# latent and its rotated key part together are one head of 256, the widest the matrix-core attention kernels take.
+MINERAX_SIZES = {
+    "2k": {"width": 2048, "heads": 16, "kv_heads": 4, "dim": 128, "rot_dim": 64, "kv_rank": 192, "window": 1024,
+           "delta_heads": 16, "delta_dim": 128, "ff": 4096, "layers": 8, "vocab": 32000},
+    "4k": {"width": 4096, "heads": 16, "kv_heads": 4, "dim": 128, "rot_dim": 64, "kv_rank": 192, "window": 2048,
+           "delta_heads": 32, "delta_dim": 128, "ff": 8192, "layers": 4, "vocab": 32000},
+}
+
+
+def minerax_config(size):
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    yarn = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot_dim"], "vdim": size["dim"],
+                        "kv_rank": size["kv_rank"], "scale": (size["dim"] + size["rot_dim"]) ** -0.5,
+                        "mask": {"size": size["window"]},
+                        "rot": {"dims": size["rot_dim"], "base": 10000.0, "scaling": yarn}}}
+    parallel = {"type": "parallel", "mlp": mlp,
+                "mixer": {"left": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"],
+                                   "vdim": size["dim"], "conv": 4, "scale": size["dim"] ** -0.5, "softcap": 50.0,
+                                   "rot": {"dims": size["dim"] // 2, "base": 10000.0, "scaling": yarn}},
+                          "right": {"heads": size["delta_heads"], "kv_heads": size["delta_heads"],
+                                    "dim": size["delta_dim"], "vdim": size["delta_dim"], "conv": 4},
+                          "left_scale": 1.0, "right_scale": 1.0}}
+    pattern = [latent, latent, latent, parallel]
+    return {"architecture": "Minerax", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+            "streams": 2, "logit_scale": size["width"] ** -0.5,
+            "layers": [pattern[i % len(pattern)] for i in range(size["layers"])]}
+
+
+def qwen3_beside_minerax(size):
+    return dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["ff"], vocab_size=size["vocab"])
+
+
 # design -> (sizes, its config at a size, Qwen3 at that size, the context a decode step may reach)
 DESIGNS = {
     "duzozen": (DUZOZEN_SIZES, duzozen_config, qwen3_beside, lambda size: 2 * size["window"]),
     "topapel": (TOPAPEL_SIZES, topapel_config, qwen3_beside_topapel, lambda size: 2 * size["chunk"]),
+    "minerax": (MINERAX_SIZES, minerax_config, qwen3_beside_minerax, lambda size: 4 * size["window"]),
 }
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
@@ -371,14 +411,14 @@ def main():
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None,
                         help="layer sizes: 8b (default), 32b, or 1.7b (the default of --workload stress)")
-    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen", "topapel"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen", "topapel", "minerax"], default="decode",
                         help="decode: the headline measurement; stress: many requests through a small cache; "
-                             "long-prompt: one long prompt in portions; duzozen, topapel: that design beside Qwen3 at "
+                             "long-prompt: one long prompt in portions; duzozen, topapel, minerax: that design beside Qwen3 at "
                              "equal sizes (--sizes), prefill and decode")
     parser.add_argument("--design-models", default="design,qwen3",
-                        help="duzozen, topapel: which of the two models to run (design: the workload's own; or its name)")
-    parser.add_argument("--design-batches", default="1,8,64", help="duzozen, topapel: the decode batch sizes to time")
-    parser.add_argument("--sizes", default="2k,4k", help="duzozen, topapel: the sizes to run, of " + ", ".join(sorted(DUZOZEN_SIZES)))
+                        help="duzozen, topapel, minerax: which of the two models to run (design: the workload's own; or its name)")
+    parser.add_argument("--design-batches", default="1,8,64", help="duzozen, topapel, minerax: the decode batch sizes to time")
+    parser.add_argument("--sizes", default="2k,4k", help="duzozen, topapel, minerax: the sizes to run, of " + ", ".join(sorted(DUZOZEN_SIZES)))
     parser.add_argument("--prompt-tokens", type=int, default=8192, help="long-prompt: tokens of the prompt")
     parser.add_argument("--portion", type=int, default=512, help="long-prompt and stress: tokens of a prompt portion (stress: also the token budget of a step)")
     parser.add_argument("--requests", type=int, default=64, help="stress: concurrent requests")

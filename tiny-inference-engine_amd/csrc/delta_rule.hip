@@ -179,26 +179,69 @@ extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int ta
 }
 
 // ---------------------------------------------------------------- the recurrence
-// A workgroup of four waves owns 64 value columns of one (sequence, value head). A lane is a column; wave p holds
-// rows [p R, (p + 1) R) of that column in registers (R = key rows a wave: a quarter of key_dim rounded up to 8,
-// 16, 32 or 64; rows beyond key_dim stay zero). The token's k, q and g lie in LDS, staged DELTA_TOKENS tokens at
-// a time (the next ones are on their way meanwhile); every lane reads the same word of them, which LDS hands to
-// a whole wave at once. The two sums over key rows (S^T k, S^T q) meet through LDS.
-#define DELTA_TOKENS 4
-#define DELTA_WAVES 4
+// One wave owns DELTA_COLS value columns of one (sequence, value head) and needs no other wave: lane l holds rows
+// [p R, (p + 1) R) of column l / 4 in registers, p = l % 4 (R = key rows a lane: a quarter of key_dim rounded up
+// to 8, 16, 32 or 64; rows beyond key_dim stay zero), so the two sums over key rows (S^T k, S^T q) meet inside a
+// quad of lanes, through two lane permutations each and without a barrier. The token's k, q and g lie in LDS,
+// staged NT tokens at a time (fewer where a lane holds more rows) (the next ones are on their way meanwhile); the lanes of one p read the
+// same words of them.
+#define DELTA_COLS 16
+
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+  return v;
+}
+
+// Where a head's columns lie inside a token's row, and where the sequence's tokens end.
+struct DeltaRowPlan {
+  int k_at, q_at, g_at, v_at, b_at, first_col, d, e, t1, row;
+};
+
+// The tokens tb .. tb + NT - 1 into registers: k, q, g of the head (padded to DP rows), then the values of the
+// wave's columns and beta.
+template <int DP, int NT, int PER, int VB>
+__device__ __forceinline__ void delta_fetch(const float* __restrict__ tok, const DeltaRowPlan pl, int tb, int lane,
+                                            float (&stage)[PER], float (&stage_vb)[VB]) {
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int idx = j * TIE_WAVE + lane;
+    const int tk = idx / (3 * DP), rest = idx % (3 * DP), which = rest / DP, i = rest % DP;
+    float v = which == 2 ? 1.f : 0.f;            // padding rows: no key, no query, no decay
+    if (tb + tk < pl.t1 && i < pl.d) {
+      const float* r = tok + static_cast<size_t>(tb + tk) * pl.row;
+      v = r[(which == 0 ? pl.k_at : (which == 1 ? pl.q_at : pl.g_at)) + i];
+    }
+    stage[j] = v;
+  }
+#pragma unroll
+  for (int j = 0; j < VB; ++j) {
+    const int idx = j * TIE_WAVE + lane;
+    const int tk = idx / (DELTA_COLS + 1), x = idx % (DELTA_COLS + 1);
+    float v = 0.f;
+    if (tk < NT && tb + tk < pl.t1) {
+      const float* r = tok + static_cast<size_t>(tb + tk) * pl.row;
+      if (x == DELTA_COLS) v = r[pl.b_at];
+      else if (pl.first_col + x < pl.e) v = r[pl.v_at + pl.first_col + x];
+    }
+    stage_vb[j] = v;
+  }
+}
 
 template <int R>
-__global__ __launch_bounds__(DELTA_WAVES* TIE_WAVE) void gated_delta_scan_kernel(
+__global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
     const float* __restrict__ tok, int row, float* __restrict__ out, int out_row, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, int G, int H, int d, int e) {
-  constexpr int DP = R * DELTA_WAVES;                 // padded key rows
-  __shared__ float kqg[DELTA_TOKENS][3][DP];
-  __shared__ float vb[DELTA_TOKENS][TIE_WAVE + 1];    // the 64 values of the columns, then beta
-  __shared__ float part[2][DELTA_WAVES][TIE_WAVE];
+  constexpr int DP = R * 4;                           // padded key rows
+  constexpr int NT = R <= 16 ? 8 : (R <= 32 ? 4 : 2);  // tokens staged at a time
+  constexpr int PER = NT * 3 * DP / TIE_WAVE;
+  constexpr int VB = (NT * (DELTA_COLS + 1) + TIE_WAVE - 1) / TIE_WAVE;
+  __shared__ float kqg[NT * 3 * DP];                  // [token][k, q, g][row]
+  __shared__ float vb[NT * (DELTA_COLS + 1)];         // [token][the values of the columns, then beta]
   const int s = blockIdx.x / H, head = blockIdx.x % H;
   const int kv = head / (H / G);
-  const int lane = threadIdx.x & (TIE_WAVE - 1), p = threadIdx.x / TIE_WAVE;
-  const int col = blockIdx.y * TIE_WAVE + lane;
+  const int lane = threadIdx.x, p = lane & 3, c = lane >> 2;
+  const int col = blockIdx.y * DELTA_COLS + c;
   const bool live = col < e;
   const int t0 = query_start[s], t1 = query_start[s + 1];
   if (t0 >= t1) return;
@@ -209,79 +252,60 @@ __global__ __launch_bounds__(DELTA_WAVES* TIE_WAVE) void gated_delta_scan_kernel
     const int i = p * R + r;
     S[r] = (live && i < d) ? sp[static_cast<size_t>(i) * e] : 0.f;
   }
-  // column offsets inside a token's row
-  const int q_at = kv * d, k_at = G * d + kv * d, v_at = 2 * G * d + head * e, b_at = 2 * G * d + H * e + head,
-            g_at = 2 * G * d + H * e + H + head * d;
-  constexpr int PER = (DELTA_TOKENS * 3 * DP + DELTA_WAVES * TIE_WAVE - 1) / (DELTA_WAVES * TIE_WAVE);
-  float stage[PER], stage_v = 0.f, stage_b = 0.f;
-
-  auto fetch = [&](int tb) {     // the tokens tb .. tb + DELTA_TOKENS - 1 into registers
+  DeltaRowPlan pl;
+  pl.q_at = kv * d;
+  pl.k_at = G * d + kv * d;
+  pl.v_at = 2 * G * d + head * e;
+  pl.b_at = 2 * G * d + H * e + head;
+  pl.g_at = 2 * G * d + H * e + H + head * d;
+  pl.first_col = blockIdx.y * DELTA_COLS;
+  pl.d = d, pl.e = e, pl.t1 = t1, pl.row = row;
+  float stage[PER], stage_vb[VB];
+  delta_fetch<DP, NT, PER, VB>(tok, pl, t0, lane, stage, stage_vb);
+  for (int tb = t0; tb < t1; tb += NT) {
+    __syncthreads();          // the wave is done with the tokens staged before
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int idx = j * (DELTA_WAVES * TIE_WAVE) + threadIdx.x;
-      const int tk = idx / (3 * DP), rest = idx % (3 * DP), which = rest / DP, i = rest % DP;
-      float v = which == 2 ? 1.f : 0.f;            // padding rows: no key, no query, no decay
-      if (tk < DELTA_TOKENS && tb + tk < t1 && i < d) {
-        const float* r = tok + static_cast<size_t>(tb + tk) * row;
-        v = r[(which == 0 ? k_at : (which == 1 ? q_at : g_at)) + i];
-      }
-      stage[j] = v;
-    }
-    // values and beta: thread (p, lane) takes token p (DELTA_TOKENS == DELTA_WAVES)
-    stage_v = stage_b = 0.f;
-    if (tb + p < t1) {
-      const float* r = tok + static_cast<size_t>(tb + p) * row;
-      stage_v = live ? r[v_at + col] : 0.f;
-      stage_b = r[b_at];
-    }
-  };
-  auto put = [&]() {
+    for (int j = 0; j < PER; ++j) kqg[j * TIE_WAVE + lane] = stage[j];
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int idx = j * (DELTA_WAVES * TIE_WAVE) + threadIdx.x;
-      if (idx < DELTA_TOKENS * 3 * DP) (&kqg[0][0][0])[idx] = stage[j];
+    for (int j = 0; j < VB; ++j) {
+      const int idx = j * TIE_WAVE + lane;
+      if (idx < NT * (DELTA_COLS + 1)) vb[idx] = stage_vb[j];
     }
-    vb[p][lane] = stage_v;
-    if (lane == 0) vb[p][TIE_WAVE] = stage_b;
-  };
-
-  fetch(t0);
-  for (int tb = t0; tb < t1; tb += DELTA_TOKENS) {
-    __syncthreads();          // everyone is done with the tokens staged before
-    put();
     __syncthreads();
-    if (tb + DELTA_TOKENS < t1) fetch(tb + DELTA_TOKENS);
-    const int count = min(DELTA_TOKENS, t1 - tb);
+    if (tb + NT < t1) delta_fetch<DP, NT, PER, VB>(tok, pl, tb + NT, lane, stage, stage_vb);
+    const int count = min(NT, t1 - tb);
     for (int j = 0; j < count; ++j) {
-      const float* kk = &kqg[j][0][p * R];
-      const float* qq = &kqg[j][1][p * R];
-      const float* gg = &kqg[j][2][p * R];
-      float dot = 0.f;
+      const float* kk = kqg + (j * 3 + 0) * DP + p * R;
+      const float* qq = kqg + (j * 3 + 1) * DP + p * R;
+      const float* gg = kqg + (j * 3 + 2) * DP + p * R;
+      float dot0 = 0.f, dot1 = 0.f, dot2 = 0.f, dot3 = 0.f;
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
+      for (int r = 0; r < R; r += 4) {
         S[r] *= gg[r];
-        dot = fmaf(S[r], kk[r], dot);
+        S[r + 1] *= gg[r + 1];
+        S[r + 2] *= gg[r + 2];
+        S[r + 3] *= gg[r + 3];
+        dot0 = fmaf(S[r], kk[r], dot0);
+        dot1 = fmaf(S[r + 1], kk[r + 1], dot1);
+        dot2 = fmaf(S[r + 2], kk[r + 2], dot2);
+        dot3 = fmaf(S[r + 3], kk[r + 3], dot3);
       }
-      part[0][p][lane] = dot;
-      __syncthreads();
-      float total = 0.f;
+      const float total = quad_sum((dot0 + dot1) + (dot2 + dot3));
+      const float u = vb[j * (DELTA_COLS + 1) + DELTA_COLS] * (vb[j * (DELTA_COLS + 1) + c] - total);
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-      for (int w = 0; w < DELTA_WAVES; ++w) total += part[0][w][lane];
-      const float u = vb[j][TIE_WAVE] * (vb[j][lane] - total);
-      float o = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
+      for (int r = 0; r < R; r += 4) {
         S[r] = fmaf(kk[r], u, S[r]);
-        o = fmaf(S[r], qq[r], o);
+        S[r + 1] = fmaf(kk[r + 1], u, S[r + 1]);
+        S[r + 2] = fmaf(kk[r + 2], u, S[r + 2]);
+        S[r + 3] = fmaf(kk[r + 3], u, S[r + 3]);
+        o0 = fmaf(S[r], qq[r], o0);
+        o1 = fmaf(S[r + 1], qq[r + 1], o1);
+        o2 = fmaf(S[r + 2], qq[r + 2], o2);
+        o3 = fmaf(S[r + 3], qq[r + 3], o3);
       }
-      part[1][p][lane] = o;
-      __syncthreads();
-      if (p == 0 && live) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < DELTA_WAVES; ++w) sum += part[1][w][lane];
-        out[static_cast<size_t>(tb + j) * out_row + head * e + col] = sum;
-      }
+      const float sum = quad_sum((o0 + o1) + (o2 + o3));
+      if (p == 0 && live) out[static_cast<size_t>(tb + j) * out_row + head * e + col] = sum;
     }
   }
 #pragma unroll
@@ -296,13 +320,12 @@ extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int o
                                     const int* query_start, const int* state_slots, int num_seqs, int G, int H, int d,
                                     int e, hipStream_t stream) {
   if (num_seqs <= 0 || G <= 0 || H <= 0 || H % G || d <= 0 || d > 256 || e <= 0 || out_row < H * e ||
-      row < 2 * G * d + H * e + H + H * d)
+      row < 2 * G * d + H * e + H + H * d || (e + DELTA_COLS - 1) / DELTA_COLS > 65535)
     return TIE_BAD_ARGUMENT;
-  const dim3 grid(num_seqs * H, (e + TIE_WAVE - 1) / TIE_WAVE);
-  const int threads = DELTA_WAVES * TIE_WAVE;
-#define SCAN(R)                                                                                                  \
-  gated_delta_scan_kernel<R><<<grid, threads, 0, stream>>>(tok, row, out, out_row, state, query_start, state_slots, \
-                                                           G, H, d, e)
+  const dim3 grid(num_seqs * H, (e + DELTA_COLS - 1) / DELTA_COLS);
+#define SCAN(R)                                                                                                   \
+  gated_delta_scan_kernel<R><<<grid, TIE_WAVE, 0, stream>>>(tok, row, out, out_row, state, query_start, state_slots, \
+                                                            G, H, d, e)
   if (d <= 32) SCAN(8);
   else if (d <= 64) SCAN(16);
   else if (d <= 128) SCAN(32);
