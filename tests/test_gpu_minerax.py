@@ -123,12 +123,13 @@ def test_rotation_with_stretched_frequencies(pairing):
     close(angles, torch.cat([torch.cos(a), torch.sin(a)], dim=1) * amplitude, 1e-5, "cos | sin")
 
 
-@pytest.mark.parametrize("H,K,N", [(3, 28, 24), (8, 64, 64), (20, 16, 48), (2, 100, 7)])
+@pytest.mark.parametrize("T", [1, 11, 200])
+@pytest.mark.parametrize("H,K,N", [(3, 28, 24), (8, 64, 64), (20, 16, 48), (2, 100, 7), (4, 192, 72), (2, 264, 200)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_a_matrix_per_head(H, K, N, dtype):
+def test_a_matrix_per_head(H, K, N, dtype, T):
+    """Sizes in and out of the steps the matrix-core kernel takes (bfloat16, K in steps of 8), few rows and many."""
     from tie_amd import kernels
 
-    T = 11
     wide = rnd(T, H, K + 8, seed=H).to(dtype).cuda()            # heads lie further apart than their width
     x = wide[:, :, :K]
     w = rnd(H, N, K, seed=K, scale=0.3).to(dtype).cuda()

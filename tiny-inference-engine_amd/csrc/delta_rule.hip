@@ -180,16 +180,19 @@ extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int ta
 
 // ---------------------------------------------------------------- the recurrence
 // One wave owns DELTA_COLS value columns of one (sequence, value head) and needs no other wave: lane l holds rows
-// [p R, (p + 1) R) of column l / 4 in registers, p = l % 4 (R = key rows a lane: a quarter of key_dim rounded up
-// to 8, 16, 32 or 64; rows beyond key_dim stay zero), so the two sums over key rows (S^T k, S^T q) meet inside a
-// quad of lanes, through two lane permutations each and without a barrier. The token's k, q and g lie in LDS,
-// staged NT tokens at a time (fewer where a lane holds more rows) (the next ones are on their way meanwhile); the lanes of one p read the
-// same words of them.
-#define DELTA_COLS 16
+// [p R, (p + 1) R) of column l / 8 in registers, p = l % 8 (R = key rows a lane: an eighth of key_dim rounded up
+// to 4, 8, 16 or 32; rows beyond key_dim stay zero), so the two sums over key rows (S^T k, S^T q) meet inside
+// eight neighbouring lanes, through three lane permutations each and without a barrier. The token's k, q and g lie
+// in LDS, staged NT tokens at a time (the next ones are on their way from memory meanwhile), every p's rows four
+// words behind the last one's so that the eight addresses of one read fall into different banks; the lanes of one
+// p read the same words. A token's words are in registers before the token before it is done.
+#define DELTA_COLS 8
+#define DELTA_PARTS 8
 
-__device__ __forceinline__ float quad_sum(float v) {
+__device__ __forceinline__ float part_sum(float v) {     // over the DELTA_PARTS lanes of a column
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));
   return v;
 }
 
@@ -228,19 +231,52 @@ __device__ __forceinline__ void delta_fetch(const float* __restrict__ tok, const
   }
 }
 
+// One token through the lane's rows: S <- g S; u = beta (v - S^T k); S <- S + k u; returns S^T q.
+template <int R>
+__device__ __forceinline__ float delta_token(float (&S)[R], const float (&kk)[R], const float (&qq)[R],
+                                             const float (&gg)[R], float v, float beta) {
+  float dot0 = 0.f, dot1 = 0.f, dot2 = 0.f, dot3 = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; r += 4) {
+    S[r] *= gg[r];
+    S[r + 1] *= gg[r + 1];
+    S[r + 2] *= gg[r + 2];
+    S[r + 3] *= gg[r + 3];
+    dot0 = fmaf(S[r], kk[r], dot0);
+    dot1 = fmaf(S[r + 1], kk[r + 1], dot1);
+    dot2 = fmaf(S[r + 2], kk[r + 2], dot2);
+    dot3 = fmaf(S[r + 3], kk[r + 3], dot3);
+  }
+  const float u = beta * (v - part_sum((dot0 + dot1) + (dot2 + dot3)));
+  float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; r += 4) {
+    S[r] = fmaf(kk[r], u, S[r]);
+    S[r + 1] = fmaf(kk[r + 1], u, S[r + 1]);
+    S[r + 2] = fmaf(kk[r + 2], u, S[r + 2]);
+    S[r + 3] = fmaf(kk[r + 3], u, S[r + 3]);
+    o0 = fmaf(S[r], qq[r], o0);
+    o1 = fmaf(S[r + 1], qq[r + 1], o1);
+    o2 = fmaf(S[r + 2], qq[r + 2], o2);
+    o3 = fmaf(S[r + 3], qq[r + 3], o3);
+  }
+  return part_sum((o0 + o1) + (o2 + o3));
+}
+
 template <int R>
 __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
     const float* __restrict__ tok, int row, float* __restrict__ out, int out_row, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, int G, int H, int d, int e) {
-  constexpr int DP = R * 4;                           // padded key rows
-  constexpr int NT = R <= 16 ? 8 : (R <= 32 ? 4 : 2);  // tokens staged at a time
+  constexpr int DP = R * DELTA_PARTS;                 // padded key rows
+  constexpr int RP = R + 4;                           // words from one p's rows to the next one's in LDS
+  constexpr int NT = R <= 16 ? 8 : 2;                 // tokens staged at a time
   constexpr int PER = NT * 3 * DP / TIE_WAVE;
   constexpr int VB = (NT * (DELTA_COLS + 1) + TIE_WAVE - 1) / TIE_WAVE;
-  __shared__ float kqg[NT * 3 * DP];                  // [token][k, q, g][row]
+  __shared__ __attribute__((aligned(16))) float kqg[NT * 3 * DELTA_PARTS * RP];   // [token][k, q, g][p][row]
   __shared__ float vb[NT * (DELTA_COLS + 1)];         // [token][the values of the columns, then beta]
   const int s = blockIdx.x / H, head = blockIdx.x % H;
   const int kv = head / (H / G);
-  const int lane = threadIdx.x, p = lane & 3, c = lane >> 2;
+  const int lane = threadIdx.x, p = lane & (DELTA_PARTS - 1), c = lane / DELTA_PARTS;
   const int col = blockIdx.y * DELTA_COLS + c;
   const bool live = col < e;
   const int t0 = query_start[s], t1 = query_start[s + 1];
@@ -262,10 +298,27 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
   pl.d = d, pl.e = e, pl.t1 = t1, pl.row = row;
   float stage[PER], stage_vb[VB];
   delta_fetch<DP, NT, PER, VB>(tok, pl, t0, lane, stage, stage_vb);
+  float ka[R], qa[R], ga[R], kb[R], qb[R], gb[R];
+  auto read = [&](int j, float (&kk)[R], float (&qq)[R], float (&gg)[R]) {     // token j of the staged ones
+    const float* at = kqg + (j * 3 * DELTA_PARTS + p) * RP;
+#pragma unroll
+    for (int r = 0; r < R; r += 4) {
+      const float4 k4 = *reinterpret_cast<const float4*>(at + r);
+      const float4 q4 = *reinterpret_cast<const float4*>(at + DELTA_PARTS * RP + r);
+      const float4 g4 = *reinterpret_cast<const float4*>(at + 2 * DELTA_PARTS * RP + r);
+      kk[r] = k4.x, kk[r + 1] = k4.y, kk[r + 2] = k4.z, kk[r + 3] = k4.w;
+      qq[r] = q4.x, qq[r + 1] = q4.y, qq[r + 2] = q4.z, qq[r + 3] = q4.w;
+      gg[r] = g4.x, gg[r + 1] = g4.y, gg[r + 2] = g4.z, gg[r + 3] = g4.w;
+    }
+  };
   for (int tb = t0; tb < t1; tb += NT) {
     __syncthreads();          // the wave is done with the tokens staged before
 #pragma unroll
-    for (int j = 0; j < PER; ++j) kqg[j * TIE_WAVE + lane] = stage[j];
+    for (int j = 0; j < PER; ++j) {
+      const int idx = j * TIE_WAVE + lane;           // [token][which][row] as fetched
+      const int i = idx % DP;
+      kqg[(idx / DP * DELTA_PARTS + i / R) * RP + i % R] = stage[j];
+    }
 #pragma unroll
     for (int j = 0; j < VB; ++j) {
       const int idx = j * TIE_WAVE + lane;
@@ -274,38 +327,26 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
     __syncthreads();
     if (tb + NT < t1) delta_fetch<DP, NT, PER, VB>(tok, pl, tb + NT, lane, stage, stage_vb);
     const int count = min(NT, t1 - tb);
-    for (int j = 0; j < count; ++j) {
-      const float* kk = kqg + (j * 3 + 0) * DP + p * R;
-      const float* qq = kqg + (j * 3 + 1) * DP + p * R;
-      const float* gg = kqg + (j * 3 + 2) * DP + p * R;
-      float dot0 = 0.f, dot1 = 0.f, dot2 = 0.f, dot3 = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; r += 4) {
-        S[r] *= gg[r];
-        S[r + 1] *= gg[r + 1];
-        S[r + 2] *= gg[r + 2];
-        S[r + 3] *= gg[r + 3];
-        dot0 = fmaf(S[r], kk[r], dot0);
-        dot1 = fmaf(S[r + 1], kk[r + 1], dot1);
-        dot2 = fmaf(S[r + 2], kk[r + 2], dot2);
-        dot3 = fmaf(S[r + 3], kk[r + 3], dot3);
+    float* o = out + static_cast<size_t>(tb) * out_row + head * e + col;
+    if constexpr (R > 16) {   // too many rows a lane for two tokens' words in registers
+      for (int j = 0; j < count; ++j) {
+        read(j, ka, qa, ga);
+        const float sum = delta_token<R>(S, ka, qa, ga, vb[j * (DELTA_COLS + 1) + c], vb[j * (DELTA_COLS + 1) + DELTA_COLS]);
+        if (p == 0 && live) o[static_cast<size_t>(j) * out_row] = sum;
       }
-      const float total = quad_sum((dot0 + dot1) + (dot2 + dot3));
-      const float u = vb[j * (DELTA_COLS + 1) + DELTA_COLS] * (vb[j * (DELTA_COLS + 1) + c] - total);
-      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
-#pragma unroll
-      for (int r = 0; r < R; r += 4) {
-        S[r] = fmaf(kk[r], u, S[r]);
-        S[r + 1] = fmaf(kk[r + 1], u, S[r + 1]);
-        S[r + 2] = fmaf(kk[r + 2], u, S[r + 2]);
-        S[r + 3] = fmaf(kk[r + 3], u, S[r + 3]);
-        o0 = fmaf(S[r], qq[r], o0);
-        o1 = fmaf(S[r + 1], qq[r + 1], o1);
-        o2 = fmaf(S[r + 2], qq[r + 2], o2);
-        o3 = fmaf(S[r + 3], qq[r + 3], o3);
+      continue;
+    }
+    read(0, ka, qa, ga);
+    for (int j = 0; j < count; j += 2) {
+      if (j + 1 < count) read(j + 1, kb, qb, gb);
+      const float first = delta_token<R>(S, ka, qa, ga, vb[j * (DELTA_COLS + 1) + c], vb[j * (DELTA_COLS + 1) + DELTA_COLS]);
+      if (p == 0 && live) o[static_cast<size_t>(j) * out_row] = first;
+      if (j + 1 < count) {
+        if (j + 2 < count) read(j + 2, ka, qa, ga);
+        const float second = delta_token<R>(S, kb, qb, gb, vb[(j + 1) * (DELTA_COLS + 1) + c],
+                                            vb[(j + 1) * (DELTA_COLS + 1) + DELTA_COLS]);
+        if (p == 0 && live) o[static_cast<size_t>(j + 1) * out_row] = second;
       }
-      const float sum = quad_sum((o0 + o1) + (o2 + o3));
-      if (p == 0 && live) out[static_cast<size_t>(tb + j) * out_row + head * e + col] = sum;
     }
   }
 #pragma unroll
@@ -326,10 +367,10 @@ extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int o
 #define SCAN(R)                                                                                                   \
   gated_delta_scan_kernel<R><<<grid, TIE_WAVE, 0, stream>>>(tok, row, out, out_row, state, query_start, state_slots, \
                                                             G, H, d, e)
-  if (d <= 32) SCAN(8);
-  else if (d <= 64) SCAN(16);
-  else if (d <= 128) SCAN(32);
-  else SCAN(64);
+  if (d <= 32) SCAN(4);
+  else if (d <= 64) SCAN(8);
+  else if (d <= 128) SCAN(16);
+  else SCAN(32);
 #undef SCAN
   return tie_launch_status();
 }

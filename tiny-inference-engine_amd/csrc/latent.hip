@@ -142,10 +142,105 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TX* __restrict__
   }
 }
 
+// The same product on the matrix cores, for bfloat16 x and w whose rows of K start at multiples of 8 elements. A
+// wave owns 16 rows x (NTILES x 16) columns of one head and reads its operands from memory in the very layout the
+// 16x16x32 instruction takes them (eight consecutive k a lane), up to 256 of K at a time, so all loads of a wave
+// are under way before its first product. Four waves a workgroup: side by side along the rows (ALONG_T, many
+// rows) or along the columns (few rows: more waves share the heads' matrices). Float32 sums.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hl_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hl_floatx4_t;
+typedef uint32_t hl_u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ hl_bf16x8_t hl_frag(hl_u32x4_t v) { return *reinterpret_cast<const hl_bf16x8_t*>(&v); }
+
+template <typename TO, int NTILES, bool ALONG_T>
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16_t* __restrict__ x, int x_row, int x_head,
+                                                               const bf16_t* __restrict__ w, TO* __restrict__ out,
+                                                               int out_row, int out_head,
+                                                               const float* __restrict__ gate, int gate_row,
+                                                               int gate_head, int T, int N, int K) {
+  const int h = blockIdx.z;
+  const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x % TIE_WAVE;
+  const int t0 = (ALONG_T ? blockIdx.x * 4 + wave : blockIdx.x) * 16;
+  const int n0 = (ALONG_T ? blockIdx.y : blockIdx.y * 4 + wave) * (NTILES * 16);
+  if (t0 >= T || n0 >= N) return;                      // the whole wave; there is no barrier below
+  const int r = lane % 16, kb = lane / 16;             // row of a fragment, block of 8 along k
+  const bf16_t* xr = x + static_cast<size_t>(min(t0 + r, T - 1)) * x_row + h * x_head + kb * 8;
+  const bf16_t* wr[NTILES];
+#pragma unroll
+  for (int i = 0; i < NTILES; ++i)
+    wr[i] = w + (static_cast<size_t>(h) * N + min(n0 + i * 16 + r, N - 1)) * K + kb * 8;
+  hl_floatx4_t acc[NTILES];
+#pragma unroll
+  for (int i = 0; i < NTILES; ++i) acc[i] = hl_floatx4_t{0.f, 0.f, 0.f, 0.f};
+  const hl_u32x4_t zero = {0u, 0u, 0u, 0u};
+  for (int k0 = 0; k0 < K; k0 += 256) {
+    hl_u32x4_t xf[8], wf[NTILES][8];
+#pragma unroll
+    for (int st = 0; st < 8; ++st) {
+      if (k0 + st * 32 >= K) continue;
+      const bool in = k0 + st * 32 + kb * 8 < K;
+      xf[st] = in ? *reinterpret_cast<const hl_u32x4_t*>(xr + k0 + st * 32) : zero;
+#pragma unroll
+      for (int i = 0; i < NTILES; ++i)
+        wf[i][st] = in ? *reinterpret_cast<const hl_u32x4_t*>(wr[i] + k0 + st * 32) : zero;
+    }
+#pragma unroll
+    for (int st = 0; st < 8; ++st) {
+      if (k0 + st * 32 >= K) continue;
+#pragma unroll
+      for (int i = 0; i < NTILES; ++i)
+        acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hl_frag(wf[i][st]), hl_frag(xf[st]), acc[i], 0, 0, 0);
+    }
+  }
+  // a lane holds row t0 + lane % 16 and, of every tile, the four columns from (lane / 16) * 4 on
+  const int t = t0 + r;
+  if (t >= T) return;
+#pragma unroll
+  for (int i = 0; i < NTILES; ++i) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int n = n0 + i * 16 + kb * 4 + v;
+      if (n >= N) continue;
+      float y = acc[i][v];
+      if (gate) y *= sigmoid_f(gate[static_cast<size_t>(t) * gate_row + h * gate_head + n]);
+      store_from_float(out + static_cast<size_t>(t) * out_row + h * out_head + n, y);
+    }
+  }
+}
+
+#define HL_FEW_ROWS 64     // up to here the four waves of a workgroup lie along the columns
+
+template <typename TO>
+static void launch_head_linear_mfma(const bf16_t* x, int x_row, int x_head, const bf16_t* w, TO* out, int out_row,
+                                    int out_head, const float* gate, int gate_row, int gate_head, int T, int H, int N,
+                                    int K, hipStream_t stream) {
+  if (T <= HL_FEW_ROWS) {
+    const dim3 grid((T + 15) / 16, (N + 63) / 64, H);
+    head_linear_mfma_kernel<TO, 1, false><<<grid, 256, 0, stream>>>(x, x_row, x_head, w, out, out_row, out_head, gate,
+                                                                    gate_row, gate_head, T, N, K);
+  } else {
+    const dim3 grid((T + 63) / 64, (N + 63) / 64, H);
+    head_linear_mfma_kernel<TO, 4, true><<<grid, 256, 0, stream>>>(x, x_row, x_head, w, out, out_row, out_head, gate,
+                                                                   gate_row, gate_head, T, N, K);
+  }
+}
+
 extern "C" int tie_head_linear(const void* x, int x_dtype, int x_row, int x_head, const void* w, int w_dtype, void* out,
                                int out_dtype, int out_row, int out_head, const float* gate, int gate_row,
                                int gate_head, int T, int H, int N, int K, hipStream_t stream) {
-  if (T <= 0 || H <= 0 || N <= 0 || K <= 0 || H > 65535) return TIE_BAD_ARGUMENT;
+  if (T <= 0 || H <= 0 || N <= 0 || K <= 0 || H > 65535 || (T + 15) / 16 > 65535 * 4) return TIE_BAD_ARGUMENT;
+  if (x_dtype == TIE_BF16 && w_dtype == TIE_BF16 && (out_dtype == TIE_BF16 || out_dtype == TIE_F32) && K % 8 == 0 &&
+      x_row % 8 == 0 && x_head % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    if (out_dtype == TIE_BF16)
+      launch_head_linear_mfma(static_cast<const bf16_t*>(x), x_row, x_head, static_cast<const bf16_t*>(w),
+                              static_cast<bf16_t*>(out), out_row, out_head, gate, gate_row, gate_head, T, H, N, K, stream);
+    else
+      launch_head_linear_mfma(static_cast<const bf16_t*>(x), x_row, x_head, static_cast<const bf16_t*>(w),
+                              static_cast<float*>(out), out_row, out_head, gate, gate_row, gate_head, T, H, N, K, stream);
+    return tie_launch_status();
+  }
   const dim3 grid((T + HL_TILE - 1) / HL_TILE, (N + HL_TILE - 1) / HL_TILE, H);
 #define HL(TX, TW, TO)                                                                                              \
   head_linear_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>(static_cast<const TX*>(x), x_row, x_head,               \

@@ -1957,7 +1957,7 @@ def hyper_connection(streams: torch.Tensor, x: Optional[torch.Tensor] = None, fr
 
 # ------------------------------------------------- short convolutions, the gated delta rule
 CONV_MAX_TAPS = 8            # CONV_MAX_TAPS of csrc/delta_rule.hip
-DELTA_RULE_MAX_DIM = 256     # key rows of a state the scan kernel keeps in registers (a quarter of them a lane)
+DELTA_RULE_MAX_DIM = 256     # key rows of a state the scan kernel keeps in registers (an eighth of them a lane)
 
 
 def conv_qkv(u: torch.Tensor, weight: torch.Tensor, taps: int, state: Optional[torch.Tensor], batch, sizes,
