@@ -79,7 +79,8 @@ extern "C" int tie_conv_qkv(const float* u, int row, const float* w, int taps, c
   if (T <= 0 || C <= 0 || taps < 1 || taps > CONV_MAX_TAPS || row < C || out_row < C ||
       static_cast<size_t>(C) * 4 > 65536 || (taps > 1 && !state))
     return TIE_BAD_ARGUMENT;
-  const int threads = C >= 4096 ? 512 : (C >= 1024 ? 256 : 128);
+  // few channels a thread: every one waits for its loads, and a decode step brings few rows
+  const int threads = C >= 2048 ? 1024 : (C >= 1024 ? 512 : (C >= 512 ? 256 : 128));
   conv_qkv_kernel<<<T, threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
       u, row, w, taps, state, state_slots, seq_of_row, query_start, nq, nk, nv, wq, wk, count_q, count_k, eps, out,
       out_row);
@@ -171,7 +172,7 @@ extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int ta
   if (T <= 0 || G <= 0 || H <= 0 || d <= 0 || e <= 0 || taps < 1 || taps > CONV_MAX_TAPS || row < C + H ||
       out_row < C + H + H * d || a_row < H * d || static_cast<size_t>(C) * 4 > 65536 || (taps > 1 && !state))
     return TIE_BAD_ARGUMENT;
-  const int threads = C >= 2048 ? 512 : 256;
+  const int threads = C >= 2048 ? 1024 : (C >= 1024 ? 512 : 256);
   delta_prepare_kernel<<<T, threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
       u, row, w, taps, state, state_slots, seq_of_row, query_start, a, a_row, A_log, dt_bias, G, H, d, e, out,
       out_row);
@@ -202,32 +203,35 @@ struct DeltaRowPlan {
 };
 
 // The tokens tb .. tb + NT - 1 into registers: k, q, g of the head (padded to DP rows), then the values of the
-// wave's columns and beta.
+// wave's columns and beta. Entry j * 64 + lane of [token][k, q, g][row]; where DP is a multiple of the wave, the
+// token and the vector of an entry are known when the kernel is compiled, and every load is issued whether it
+// counts or not (from an address that exists), so that none waits for a branch.
 template <int DP, int NT, int PER, int VB>
 __device__ __forceinline__ void delta_fetch(const float* __restrict__ tok, const DeltaRowPlan pl, int tb, int lane,
                                             float (&stage)[PER], float (&stage_vb)[VB]) {
+  const float* first = tok + static_cast<size_t>(tb) * pl.row;
+  const int left = pl.t1 - tb;                    // tokens from tb on, at least one
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const int idx = j * TIE_WAVE + lane;
-    const int tk = idx / (3 * DP), rest = idx % (3 * DP), which = rest / DP, i = rest % DP;
-    float v = which == 2 ? 1.f : 0.f;            // padding rows: no key, no query, no decay
-    if (tb + tk < pl.t1 && i < pl.d) {
-      const float* r = tok + static_cast<size_t>(tb + tk) * pl.row;
-      v = r[(which == 0 ? pl.k_at : (which == 1 ? pl.q_at : pl.g_at)) + i];
+    int tk, which, i;
+    if constexpr (DP % TIE_WAVE == 0) {
+      tk = j * TIE_WAVE / (3 * DP), which = j * TIE_WAVE % (3 * DP) / DP, i = j * TIE_WAVE % DP + lane;
+    } else {
+      const int idx = j * TIE_WAVE + lane, rest = idx % (3 * DP);
+      tk = idx / (3 * DP), which = rest / DP, i = rest % DP;
     }
-    stage[j] = v;
+    const float* r = first + static_cast<size_t>(min(tk, left - 1)) * pl.row;
+    const float v = r[(which == 0 ? pl.k_at : (which == 1 ? pl.q_at : pl.g_at)) + min(i, pl.d - 1)];
+    stage[j] = (tk < left && i < pl.d) ? v : (which == 2 ? 1.f : 0.f);     // padding: no key, no query, no decay
   }
 #pragma unroll
   for (int j = 0; j < VB; ++j) {
     const int idx = j * TIE_WAVE + lane;
     const int tk = idx / (DELTA_COLS + 1), x = idx % (DELTA_COLS + 1);
-    float v = 0.f;
-    if (tk < NT && tb + tk < pl.t1) {
-      const float* r = tok + static_cast<size_t>(tb + tk) * pl.row;
-      if (x == DELTA_COLS) v = r[pl.b_at];
-      else if (pl.first_col + x < pl.e) v = r[pl.v_at + pl.first_col + x];
-    }
-    stage_vb[j] = v;
+    const float* r = first + static_cast<size_t>(min(tk, left - 1)) * pl.row;
+    const int col = min(pl.first_col + x, pl.e - 1);
+    const float v = r[x == DELTA_COLS ? pl.b_at : pl.v_at + col];
+    stage_vb[j] = (tk < NT && tk < left && (x == DELTA_COLS || pl.first_col + x < pl.e)) ? v : 0.f;
   }
 }
 
@@ -314,10 +318,14 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
   for (int tb = t0; tb < t1; tb += NT) {
     __syncthreads();          // the wave is done with the tokens staged before
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-      const int idx = j * TIE_WAVE + lane;           // [token][which][row] as fetched
-      const int i = idx % DP;
-      kqg[(idx / DP * DELTA_PARTS + i / R) * RP + i % R] = stage[j];
+    for (int j = 0; j < PER; ++j) {                  // [token][which][row] as fetched
+      int vec, i;
+      if constexpr (DP % TIE_WAVE == 0) {
+        vec = j * TIE_WAVE / DP, i = j * TIE_WAVE % DP + lane;
+      } else {
+        vec = (j * TIE_WAVE + lane) / DP, i = (j * TIE_WAVE + lane) % DP;
+      }
+      kqg[(vec * DELTA_PARTS + i / R) * RP + i % R] = stage[j];
     }
 #pragma unroll
     for (int j = 0; j < VB; ++j) {
