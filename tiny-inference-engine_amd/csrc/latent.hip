@@ -144,8 +144,9 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TX* __restrict__
 
 // The same product on the matrix cores, for bfloat16 x and w whose rows of K start at multiples of 8 elements. A
 // wave owns 16 rows x (NTILES x 16) columns of one head and reads its operands from memory in the very layout the
-// 16x16x32 instruction takes them (eight consecutive k a lane), up to 256 of K at a time, so all loads of a wave
-// are under way before its first product. Four waves a workgroup: side by side along the rows (ALONG_T, many
+// 16x16x32 instruction takes them (eight consecutive k a lane), KSTEPS x 32 of K at a time, so those loads of a wave
+// are under way before its first product. A lane ends with four consecutive columns of one row a tile, stored as one
+// word where the sizes allow. Four waves a workgroup: side by side along the rows (ALONG_T, many
 // rows) or along the columns (few rows: more waves share the heads' matrices). Float32 sums.
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hl_bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hl_floatx4_t;
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16_t* __r
                                                                const bf16_t* __restrict__ w, TO* __restrict__ out,
                                                                int out_row, int out_head,
                                                                const float* __restrict__ gate, int gate_row,
-                                                               int gate_head, int T, int N, int K) {
+                                                               int gate_head, int T, int N, int K, int whole) {
   const int h = blockIdx.z;
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x % TIE_WAVE;
   const int t0 = (ALONG_T ? blockIdx.x * 4 + wave : blockIdx.x) * 16;
@@ -174,10 +175,11 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16_t* __r
 #pragma unroll
   for (int i = 0; i < NTILES; ++i) acc[i] = hl_floatx4_t{0.f, 0.f, 0.f, 0.f};
   const hl_u32x4_t zero = {0u, 0u, 0u, 0u};
-  for (int k0 = 0; k0 < K; k0 += 256) {
-    hl_u32x4_t xf[8], wf[NTILES][8];
+  constexpr int KSTEPS = NTILES == 1 ? 8 : 4;
+  for (int k0 = 0; k0 < K; k0 += KSTEPS * 32) {
+    hl_u32x4_t xf[KSTEPS], wf[NTILES][KSTEPS];
 #pragma unroll
-    for (int st = 0; st < 8; ++st) {
+    for (int st = 0; st < KSTEPS; ++st) {
       if (k0 + st * 32 >= K) continue;
       const bool in = k0 + st * 32 + kb * 8 < K;
       xf[st] = in ? *reinterpret_cast<const hl_u32x4_t*>(xr + k0 + st * 32) : zero;
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16_t* __r
         wf[i][st] = in ? *reinterpret_cast<const hl_u32x4_t*>(wr[i] + k0 + st * 32) : zero;
     }
 #pragma unroll
-    for (int st = 0; st < 8; ++st) {
+    for (int st = 0; st < KSTEPS; ++st) {
       if (k0 + st * 32 >= K) continue;
 #pragma unroll
       for (int i = 0; i < NTILES; ++i)
@@ -198,13 +200,32 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(const bf16_t* __r
   if (t >= T) return;
 #pragma unroll
   for (int i = 0; i < NTILES; ++i) {
+    const int n = n0 + i * 16 + kb * 4;
+    if (n >= N) continue;
+    TO* o = out + static_cast<size_t>(t) * out_row + h * out_head + n;
+    const float* g = gate ? gate + static_cast<size_t>(t) * gate_row + h * gate_head + n : nullptr;
+    if (whole) {           // n + 3 < N, and four columns are one aligned word of out (and of gate)
+      float y[4] = {acc[i][0], acc[i][1], acc[i][2], acc[i][3]};
+      if (g) {
+        const float4 g4 = *reinterpret_cast<const float4*>(g);
+        y[0] *= sigmoid_f(g4.x), y[1] *= sigmoid_f(g4.y), y[2] *= sigmoid_f(g4.z), y[3] *= sigmoid_f(g4.w);
+      }
+      if constexpr (sizeof(TO) == 2) {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(float_to_bf16(y[0])) | (static_cast<uint32_t>(float_to_bf16(y[1])) << 16);
+        packed.y = static_cast<uint32_t>(float_to_bf16(y[2])) | (static_cast<uint32_t>(float_to_bf16(y[3])) << 16);
+        *reinterpret_cast<uint2*>(o) = packed;
+      } else {
+        *reinterpret_cast<float4*>(o) = make_float4(y[0], y[1], y[2], y[3]);
+      }
+      continue;
+    }
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      const int n = n0 + i * 16 + kb * 4 + v;
-      if (n >= N) continue;
+      if (n + v >= N) continue;
       float y = acc[i][v];
-      if (gate) y *= sigmoid_f(gate[static_cast<size_t>(t) * gate_row + h * gate_head + n]);
-      store_from_float(out + static_cast<size_t>(t) * out_row + h * out_head + n, y);
+      if (g) y *= sigmoid_f(g[v]);
+      store_from_float(o + v, y);
     }
   }
 }
@@ -215,14 +236,18 @@ template <typename TO>
 static void launch_head_linear_mfma(const bf16_t* x, int x_row, int x_head, const bf16_t* w, TO* out, int out_row,
                                     int out_head, const float* gate, int gate_row, int gate_head, int T, int H, int N,
                                     int K, hipStream_t stream) {
+  // four columns a store (and a gate load): sizes in steps of four from aligned addresses
+  const int whole = N % 4 == 0 && out_row % 4 == 0 && out_head % 4 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % (4 * sizeof(TO)) == 0 &&
+                    (!gate || (gate_row % 4 == 0 && gate_head % 4 == 0 && reinterpret_cast<uintptr_t>(gate) % 16 == 0));
   if (T <= HL_FEW_ROWS) {
     const dim3 grid((T + 15) / 16, (N + 63) / 64, H);
     head_linear_mfma_kernel<TO, 1, false><<<grid, 256, 0, stream>>>(x, x_row, x_head, w, out, out_row, out_head, gate,
-                                                                    gate_row, gate_head, T, N, K);
+                                                                    gate_row, gate_head, T, N, K, whole);
   } else {
     const dim3 grid((T + 63) / 64, (N + 63) / 64, H);
     head_linear_mfma_kernel<TO, 4, true><<<grid, 256, 0, stream>>>(x, x_row, x_head, w, out, out_row, out_head, gate,
-                                                                   gate_row, gate_head, T, N, K);
+                                                                   gate_row, gate_head, T, N, K, whole);
   }
 }
 
