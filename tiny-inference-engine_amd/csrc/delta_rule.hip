@@ -124,7 +124,7 @@ extern "C" int tie_conv_state_update(const float* u, int row, int taps, float* s
 
 // ---------------------------------------------------------------- what the delta rule takes of a token
 // Row t of `u`: [q (G d) | k (G d) | v (H e) | b (H)], the first C = 2 G d + H e columns convolved, then silu.
-// Row t of `a`: the decay's argument (H d), `a_row` apart. out row: [q^ | k^ | v | beta (H) | g (H d)]:
+// Row t of `a`: the decay's argument (H d), `a_row` apart. out row: [q^ | k^ | v | g (H d) | beta (H)]:
 //   q^, k^ unit vectors per head (x / sqrt(sum x^2 + 1e-6)), q^ also times d^(-1/2); beta = sigmoid(b);
 //   g = exp(-exp(A_log[head]) * softplus(a + dt_bias)).
 __global__ void delta_prepare_kernel(const float* __restrict__ u, int row, const float* __restrict__ w, int taps,
@@ -158,10 +158,10 @@ __global__ void delta_prepare_kernel(const float* __restrict__ u, int row, const
   }
   for (int c = 2 * G * d + threadIdx.x; c < C; c += blockDim.x) o[c] = vals[c];
   const float* b = u + static_cast<size_t>(t) * row + C;
-  for (int h = threadIdx.x; h < H; h += blockDim.x) o[C + h] = sigmoid_f(b[h]);
+  for (int h = threadIdx.x; h < H; h += blockDim.x) o[C + H * d + h] = sigmoid_f(b[h]);
   const float* ar = a + static_cast<size_t>(t) * a_row;
   for (int c = threadIdx.x; c < H * d; c += blockDim.x)
-    o[C + H + c] = expf(-expf(A_log[c / d]) * softplus_f(ar[c] + dt_bias[c]));
+    o[C + c] = expf(-expf(A_log[c / d]) * softplus_f(ar[c] + dt_bias[c]));
 }
 
 extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int taps, const float* state,
@@ -180,15 +180,18 @@ extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int ta
 }
 
 // ---------------------------------------------------------------- the recurrence
-// One wave owns DELTA_COLS value columns of one (sequence, value head) and needs no other wave: lane l holds rows
-// [p R, (p + 1) R) of column l / 8 in registers, p = l % 8 (R = key rows a lane: an eighth of key_dim rounded up
-// to 4, 8, 16 or 32; rows beyond key_dim stay zero), so the two sums over key rows (S^T k, S^T q) meet inside
-// eight neighbouring lanes, through three lane permutations each and without a barrier. The token's k, q and g lie
-// in LDS, staged NT tokens at a time (the next ones are on their way from memory meanwhile), every p's rows four
-// words behind the last one's so that the eight addresses of one read fall into different banks; the lanes of one
-// p read the same words. A token's words are in registers before the token before it is done.
+// A wave owns DELTA_COLS value columns of one (sequence, value head): lane l holds rows [p R, (p + 1) R) of column
+// l / 8 in registers, p = l % 8 (R = key rows a lane: an eighth of key_dim rounded up to 4, 8, 16 or 32; rows
+// beyond key_dim stay zero), so the two sums over key rows (S^T k, S^T q) meet inside eight neighbouring lanes,
+// through three lane permutations each and without a barrier. The DELTA_WAVES waves of a workgroup take columns
+// side by side and share the token's k, q and g in LDS, staged NT tokens at a time (the next ones are on their way
+// from memory meanwhile, four words a load where the row's layout allows), every p's rows four words behind the
+// last one's so that the eight addresses of one read fall into different banks; the lanes of one p read the same
+// words. A token's words are in registers before the token before it is done.
 #define DELTA_COLS 8
 #define DELTA_PARTS 8
+#define DELTA_WAVES 4
+#define DELTA_THREADS (DELTA_WAVES * TIE_WAVE)
 
 __device__ __forceinline__ float part_sum(float v) {     // over the DELTA_PARTS lanes of a column
   v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));
@@ -202,35 +205,44 @@ struct DeltaRowPlan {
   int k_at, q_at, g_at, v_at, b_at, first_col, d, e, t1, row;
 };
 
-// The tokens tb .. tb + NT - 1 into registers: k, q, g of the head (padded to DP rows), then the values of the
-// wave's columns and beta. Entry j * 64 + lane of [token][k, q, g][row]; where DP is a multiple of the wave, the
-// token and the vector of an entry are known when the kernel is compiled, and every load is issued whether it
-// counts or not (from an address that exists), so that none waits for a branch.
-template <int DP, int NT, int PER, int VB>
-__device__ __forceinline__ void delta_fetch(const float* __restrict__ tok, const DeltaRowPlan pl, int tb, int lane,
-                                            float (&stage)[PER], float (&stage_vb)[VB]) {
+// k, q and g of the tokens tb .. tb + NT - 1 of the head (padded to DP rows) into registers, W words a load:
+// entry (x * DELTA_THREADS + thread) * W of [token][k, q, g][row]. Every load is issued whether it counts or not
+// (from an address that exists), so that none waits for a branch.
+template <int DP, int NT, int W, int PER>
+__device__ __forceinline__ void delta_fetch(const float* __restrict__ tok, const DeltaRowPlan pl, int tb,
+                                            float (&stage)[PER][W]) {
   const float* first = tok + static_cast<size_t>(tb) * pl.row;
   const int left = pl.t1 - tb;                    // tokens from tb on, at least one
 #pragma unroll
-  for (int j = 0; j < PER; ++j) {
-    int tk, which, i;
-    if constexpr (DP % TIE_WAVE == 0) {
-      tk = j * TIE_WAVE / (3 * DP), which = j * TIE_WAVE % (3 * DP) / DP, i = j * TIE_WAVE % DP + lane;
+  for (int x = 0; x < PER; ++x) {
+    const int idx = (x * DELTA_THREADS + static_cast<int>(threadIdx.x)) * W;
+    const int tk = idx / (3 * DP), rest = idx % (3 * DP), which = rest / DP, i = rest % DP;
+    const float* r = first + static_cast<size_t>(min(tk, left - 1)) * pl.row +
+                     (which == 0 ? pl.k_at : (which == 1 ? pl.q_at : pl.g_at));
+    const float pad = which == 2 ? 1.f : 0.f;      // padding rows: no key, no query, no decay
+    if constexpr (W == 4) {                        // d is a multiple of 4: the four rows count together
+      const float4 v = *reinterpret_cast<const float4*>(r + min(i, pl.d - 4));
+      const bool in = tk < left && i < pl.d;
+      stage[x][0] = in ? v.x : pad, stage[x][1] = in ? v.y : pad, stage[x][2] = in ? v.z : pad, stage[x][3] = in ? v.w : pad;
     } else {
-      const int idx = j * TIE_WAVE + lane, rest = idx % (3 * DP);
-      tk = idx / (3 * DP), which = rest / DP, i = rest % DP;
+      const float v = r[min(i, pl.d - 1)];
+      stage[x][0] = (tk < left && i < pl.d) ? v : pad;
     }
-    const float* r = first + static_cast<size_t>(min(tk, left - 1)) * pl.row;
-    const float v = r[(which == 0 ? pl.k_at : (which == 1 ? pl.q_at : pl.g_at)) + min(i, pl.d - 1)];
-    stage[j] = (tk < left && i < pl.d) ? v : (which == 2 ? 1.f : 0.f);     // padding: no key, no query, no decay
   }
+}
+
+// The values of the wave's columns and beta of the same tokens: entry j * 64 + lane of [token][columns, beta].
+template <int NT, int VB>
+__device__ __forceinline__ void delta_fetch_values(const float* __restrict__ tok, const DeltaRowPlan pl, int tb,
+                                                   int lane, float (&stage_vb)[VB]) {
+  const float* first = tok + static_cast<size_t>(tb) * pl.row;
+  const int left = pl.t1 - tb;
 #pragma unroll
   for (int j = 0; j < VB; ++j) {
     const int idx = j * TIE_WAVE + lane;
     const int tk = idx / (DELTA_COLS + 1), x = idx % (DELTA_COLS + 1);
     const float* r = first + static_cast<size_t>(min(tk, left - 1)) * pl.row;
-    const int col = min(pl.first_col + x, pl.e - 1);
-    const float v = r[x == DELTA_COLS ? pl.b_at : pl.v_at + col];
+    const float v = r[x == DELTA_COLS ? pl.b_at : pl.v_at + min(pl.first_col + x, pl.e - 1)];
     stage_vb[j] = (tk < NT && tk < left && (x == DELTA_COLS || pl.first_col + x < pl.e)) ? v : 0.f;
   }
 }
@@ -267,24 +279,26 @@ __device__ __forceinline__ float delta_token(float (&S)[R], const float (&kk)[R]
   return part_sum((o0 + o1) + (o2 + o3));
 }
 
-template <int R>
-__global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
+template <int R, int W>
+__global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
     const float* __restrict__ tok, int row, float* __restrict__ out, int out_row, float* __restrict__ state,
     const int* __restrict__ query_start, const int* __restrict__ state_slots, int G, int H, int d, int e) {
   constexpr int DP = R * DELTA_PARTS;                 // padded key rows
   constexpr int RP = R + 4;                           // words from one p's rows to the next one's in LDS
-  constexpr int NT = R <= 16 ? 8 : 2;                 // tokens staged at a time
-  constexpr int PER = NT * 3 * DP / TIE_WAVE;
+  constexpr int NT = 4 * DELTA_THREADS / DP;          // tokens staged at a time: 4 to 32
+  constexpr int PER = NT * 3 * DP / (DELTA_THREADS * W);
   constexpr int VB = (NT * (DELTA_COLS + 1) + TIE_WAVE - 1) / TIE_WAVE;
   __shared__ __attribute__((aligned(16))) float kqg[NT * 3 * DELTA_PARTS * RP];   // [token][k, q, g][p][row]
-  __shared__ float vb[NT * (DELTA_COLS + 1)];         // [token][the values of the columns, then beta]
+  __shared__ float vbs[DELTA_WAVES][NT * (DELTA_COLS + 1)];     // a wave: [token][the values of its columns, beta]
   const int s = blockIdx.x / H, head = blockIdx.x % H;
   const int kv = head / (H / G);
-  const int lane = threadIdx.x, p = lane & (DELTA_PARTS - 1), c = lane / DELTA_PARTS;
-  const int col = blockIdx.y * DELTA_COLS + c;
+  const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x % TIE_WAVE;
+  const int p = lane & (DELTA_PARTS - 1), c = lane / DELTA_PARTS;
+  const int first_col = (blockIdx.y * DELTA_WAVES + wave) * DELTA_COLS;
+  const int col = first_col + c;
   const bool live = col < e;
   const int t0 = query_start[s], t1 = query_start[s + 1];
-  if (t0 >= t1) return;
+  if (t0 >= t1) return;                               // the whole workgroup
   float* sp = state + ((static_cast<size_t>(state_slots[s]) * H + head) * d) * e + col;
   float S[R];
 #pragma unroll
@@ -296,12 +310,14 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
   pl.q_at = kv * d;
   pl.k_at = G * d + kv * d;
   pl.v_at = 2 * G * d + head * e;
-  pl.b_at = 2 * G * d + H * e + head;
-  pl.g_at = 2 * G * d + H * e + H + head * d;
-  pl.first_col = blockIdx.y * DELTA_COLS;
+  pl.g_at = 2 * G * d + H * e + head * d;
+  pl.b_at = 2 * G * d + H * e + H * d + head;
+  pl.first_col = first_col;
   pl.d = d, pl.e = e, pl.t1 = t1, pl.row = row;
-  float stage[PER], stage_vb[VB];
-  delta_fetch<DP, NT, PER, VB>(tok, pl, t0, lane, stage, stage_vb);
+  float* vb = vbs[wave];
+  float stage[PER][W], stage_vb[VB];
+  delta_fetch<DP, NT, W, PER>(tok, pl, t0, stage);
+  delta_fetch_values<NT, VB>(tok, pl, t0, lane, stage_vb);
   float ka[R], qa[R], ga[R], kb[R], qb[R], gb[R];
   auto read = [&](int j, float (&kk)[R], float (&qq)[R], float (&gg)[R]) {     // token j of the staged ones
     const float* at = kqg + (j * 3 * DELTA_PARTS + p) * RP;
@@ -316,16 +332,17 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
     }
   };
   for (int tb = t0; tb < t1; tb += NT) {
-    __syncthreads();          // the wave is done with the tokens staged before
+    __syncthreads();          // every wave is done with the tokens staged before
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {                  // [token][which][row] as fetched
-      int vec, i;
-      if constexpr (DP % TIE_WAVE == 0) {
-        vec = j * TIE_WAVE / DP, i = j * TIE_WAVE % DP + lane;
+    for (int x = 0; x < PER; ++x) {                  // [token][which][row] as fetched
+      const int idx = (x * DELTA_THREADS + static_cast<int>(threadIdx.x)) * W;
+      const int vec = idx / DP, i = idx % DP;
+      float* to = kqg + (vec * DELTA_PARTS + i / R) * RP + i % R;
+      if constexpr (W == 4) {
+        *reinterpret_cast<float4*>(to) = make_float4(stage[x][0], stage[x][1], stage[x][2], stage[x][3]);
       } else {
-        vec = (j * TIE_WAVE + lane) / DP, i = (j * TIE_WAVE + lane) % DP;
+        *to = stage[x][0];
       }
-      kqg[(vec * DELTA_PARTS + i / R) * RP + i % R] = stage[j];
     }
 #pragma unroll
     for (int j = 0; j < VB; ++j) {
@@ -333,7 +350,10 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
       if (idx < NT * (DELTA_COLS + 1)) vb[idx] = stage_vb[j];
     }
     __syncthreads();
-    if (tb + NT < t1) delta_fetch<DP, NT, PER, VB>(tok, pl, tb + NT, lane, stage, stage_vb);
+    if (tb + NT < t1) {
+      delta_fetch<DP, NT, W, PER>(tok, pl, tb + NT, stage);
+      delta_fetch_values<NT, VB>(tok, pl, tb + NT, lane, stage_vb);
+    }
     const int count = min(NT, t1 - tb);
     float* o = out + static_cast<size_t>(tb) * out_row + head * e + col;
     if constexpr (R > 16) {   // too many rows a lane for two tokens' words in registers
@@ -368,13 +388,22 @@ __global__ __launch_bounds__(TIE_WAVE) void gated_delta_scan_kernel(
 extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int out_row, float* state,
                                     const int* query_start, const int* state_slots, int num_seqs, int G, int H, int d,
                                     int e, hipStream_t stream) {
+  constexpr int wg_cols = DELTA_WAVES * DELTA_COLS;
   if (num_seqs <= 0 || G <= 0 || H <= 0 || H % G || d <= 0 || d > 256 || e <= 0 || out_row < H * e ||
-      row < 2 * G * d + H * e + H + H * d || (e + DELTA_COLS - 1) / DELTA_COLS > 65535)
+      row < 2 * G * d + H * e + H + H * d || (e + wg_cols - 1) / wg_cols > 65535)
     return TIE_BAD_ARGUMENT;
-  const dim3 grid(num_seqs * H, (e + DELTA_COLS - 1) / DELTA_COLS);
-#define SCAN(R)                                                                                                   \
-  gated_delta_scan_kernel<R><<<grid, TIE_WAVE, 0, stream>>>(tok, row, out, out_row, state, query_start, state_slots, \
-                                                            G, H, d, e)
+  const dim3 grid(num_seqs * H, (e + wg_cols - 1) / wg_cols);
+  // four words a load where every head's k, q and g start at a multiple of four words of an aligned row
+  const bool wide = d % 4 == 0 && (H * e) % 4 == 0 && row % 4 == 0 && reinterpret_cast<uintptr_t>(tok) % 16 == 0;
+#define SCAN(R)                                                                                                    \
+  do {                                                                                                             \
+    if (wide)                                                                                                      \
+      gated_delta_scan_kernel<R, 4><<<grid, DELTA_THREADS, 0, stream>>>(tok, row, out, out_row, state, query_start, \
+                                                                        state_slots, G, H, d, e);                   \
+    else                                                                                                           \
+      gated_delta_scan_kernel<R, 1><<<grid, DELTA_THREADS, 0, stream>>>(tok, row, out, out_row, state, query_start, \
+                                                                        state_slots, G, H, d, e);                   \
+  } while (0)
   if (d <= 32) SCAN(4);
   else if (d <= 64) SCAN(8);
   else if (d <= 128) SCAN(16);

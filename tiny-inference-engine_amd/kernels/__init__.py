@@ -2023,7 +2023,7 @@ def delta_prepare(u: torch.Tensor, weight: torch.Tensor, taps: int, state: Optio
 
     ``u`` rows ``[q (G d) | k (G d) | v (H e) | b (H)]``: q, k, v through the short convolution and silu, q and k
     made unit vectors per head (q also times ``d ** -0.5``), ``beta = sigmoid(b)``; ``a`` rows ``[H d]``: the decays
-    ``exp(-exp(A_log[head]) * softplus(a + dt_bias))``. ``out`` rows: ``[q | k | v | beta | decay]`` float32."""
+    ``exp(-exp(A_log[head]) * softplus(a + dt_bias))``. ``out`` rows: ``[q | k | v | decay | beta]`` float32."""
     G, H, d, e = kv_heads, heads, key_dim, value_dim
     C = 2 * G * d + H * e
     _gpu_strided(u, "projected rows")
