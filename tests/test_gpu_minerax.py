@@ -180,11 +180,36 @@ def test_short_convolution_and_the_norm_over_a_projection(taps):
         close(torch.cat(got[s]), want[s], 3e-6, f"sequence {s}, {taps} taps")
 
 
+def chunks_of(counts, rows):
+    """A step's rows cut into chunks of at most ``rows``, as the engine hands them to the kernels."""
+    from tie_amd import kernels
+
+    items, first, row = [], [0], 0
+    for s, n in enumerate(counts):
+        pieces = -(-n // rows)
+        items += [(s, row + n * i // pieces, row + n * (i + 1) // pieces) for i in range(pieces)]
+        row += n
+        first.append(len(items))
+    return kernels.ScanChunks(i32(items), i32(first), len(items), max(b - a for _, a, b in items))
+
+
+class Scratch:
+    def __init__(self):
+        self.memory = {}
+
+    def __call__(self, name, shape, dtype):
+        key = (name, tuple(shape), dtype)
+        if key not in self.memory:
+            self.memory[key] = torch.full(tuple(shape), float("nan"), dtype=dtype, device="cuda")
+        return self.memory[key]
+
+
+@pytest.mark.parametrize("chunk_rows", [None, 1, 3, 7])
 @pytest.mark.parametrize("G,H,d,e,taps", [(2, 4, 8, 24, 3), (1, 1, 32, 64, 4), (2, 2, 40, 16, 2), (1, 3, 20, 9, 1),
                                           (2, 2, 64, 80, 3), (1, 2, 128, 128, 4), (1, 1, 200, 70, 2)])
-def test_gated_delta_rule_kernels(G, H, d, e, taps):
+def test_gated_delta_rule_kernels(G, H, d, e, taps, chunk_rows):
     """Rows of projections -> convolution, silu, unit vectors, beta, decays -> the recurrence, sequences cut anywhere
-    and states in slots that are not in order; then the gated norm of the heads."""
+    and states in slots that are not in order, whole or chunk beside chunk; then the gated norm of the heads."""
     from tie_amd import kernels
 
     silu = torch.nn.functional.silu
@@ -221,7 +246,8 @@ def test_gated_delta_rule_kernels(G, H, d, e, taps):
         if taps > 1:
             kernels.conv_state_update(rows, taps, conv_state, batch, C)
         out = torch.empty(T, H * e, device="cuda")
-        kernels.gated_delta_scan(tok, out, state, batch, G, H, d, e)
+        chunks = chunks_of([n for _, n in step], chunk_rows) if chunk_rows else None
+        kernels.gated_delta_scan(tok, out, state, batch, G, H, d, e, chunks=chunks, scratch=Scratch())
         r = 0
         for s, n in step:
             got[s].append(out[r:r + n].cpu())
@@ -462,6 +488,37 @@ def test_long_decoding_through_windows_with_pages_given_back_and_used_again(fold
     got = th.collect(rep, steps)
     assert rep.cache.all_free()
     check(got, want, TOLERANCE["float32"], "long decoding")
+
+
+def test_long_portions_run_the_delta_rule_chunk_beside_chunk(folders, monkeypatch):
+    """Portions long enough for the three-launch walk (made to start at fewer rows here, in smaller chunks), beside a
+    short one and a single token, against the plain model and against the same requests in short portions."""
+    from tie_amd import kernels
+    from tie_amd.engine.replay import TraceReplayer
+
+    monkeypatch.setattr(kernels, "DELTA_CHUNKS_FROM", 400)
+    monkeypatch.setattr(kernels, "DELTA_CHUNK_ROWS", 96)
+    folder, config = folders["D", "float32"], CONFIGS["D"]
+    requests = th.make_requests(config["vocab"], [700, 560, 40], seed=17)
+    want = reference(folder, config, requests)
+    a, b, c = requests["r0"], requests["r1"], requests["r2"]
+    steps = [
+        {"step": 0, "entries": [{"id": "r2", "tokens": c[:39], "want": list(range(39))}], "end": []},
+        {"step": 1, "entries": [{"id": "r0", "tokens": a[:670], "want": list(range(670))},
+                                {"id": "r2", "tokens": c[39:], "want": [0]},
+                                {"id": "r1", "tokens": b[:10], "want": list(range(10))}], "end": ["r2"]},
+        {"step": 2, "entries": [{"id": "r1", "tokens": b[10:], "want": list(range(550))},
+                                {"id": "r0", "tokens": a[670:], "want": list(range(30))}], "end": ["r0", "r1"]},
+    ]
+    rep = TraceReplayer.from_folder(folder, "float32", 1408, block_size=BLOCK_SIZE["D"])
+    got = th.collect(rep, steps)
+    assert rep.cache.all_free()
+    check(got, want, TOLERANCE["float32"], "long portions")
+    short = th.collect(TraceReplayer.from_folder(folder, "float32", 1408, block_size=BLOCK_SIZE["D"]),
+                       th.portions({"r0": a}, sizes=(97, 150, 33)))
+    mine = torch.stack([got["r0"][p] for p in range(len(a))])
+    other = torch.stack([short["r0"][p] for p in range(len(a))])
+    assert float((mine - other).abs().max() / mine.abs().max()) < 1e-5
 
 
 def test_state_slots_are_cleared_when_they_are_used_again(folders):

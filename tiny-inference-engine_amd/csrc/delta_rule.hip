@@ -279,10 +279,24 @@ __device__ __forceinline__ float delta_token(float (&S)[R], const float (&kk)[R]
   return part_sum((o0 + o1) + (o2 + o3));
 }
 
+// What a launch of the scan walks. Without `items` a workgroup's rows are a sequence's rows of the step and its
+// state the sequence's slot. With `items` ([count][3]: sequence, first row, end row) they are one chunk's, and the
+// state is entry `item` of `state`. A state has `columns` columns: e, or e + d where the columns from e on carry the
+// chunk's transition (they start as the identity and take no values, so they end as the product of the tokens'
+// transition matrices, which is what the state before the chunk is multiplied by).
+struct DeltaScanMode {
+  const int* items;
+  int columns;
+  int init;      // 0: the state is read; 1: it starts as zeros (and the identity from column e on)
+  int store;     // the state is written back at the end
+  int outputs;   // outputs are written
+};
+
 template <int R, int W>
 __global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
     const float* __restrict__ tok, int row, float* __restrict__ out, int out_row, float* __restrict__ state,
-    const int* __restrict__ query_start, const int* __restrict__ state_slots, int G, int H, int d, int e) {
+    const int* __restrict__ query_start, const int* __restrict__ state_slots, int G, int H, int d, int e,
+    DeltaScanMode mode) {
   constexpr int DP = R * DELTA_PARTS;                 // padded key rows
   constexpr int RP = R + 4;                           // words from one p's rows to the next one's in LDS
   constexpr int NT = 4 * DELTA_THREADS / DP;          // tokens staged at a time: 4 to 32
@@ -290,21 +304,28 @@ __global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
   constexpr int VB = (NT * (DELTA_COLS + 1) + TIE_WAVE - 1) / TIE_WAVE;
   __shared__ __attribute__((aligned(16))) float kqg[NT * 3 * DELTA_PARTS * RP];   // [token][k, q, g][p][row]
   __shared__ float vbs[DELTA_WAVES][NT * (DELTA_COLS + 1)];     // a wave: [token][the values of its columns, beta]
-  const int s = blockIdx.x / H, head = blockIdx.x % H;
+  const int item = blockIdx.x / H, head = blockIdx.x % H;
   const int kv = head / (H / G);
   const int wave = threadIdx.x / TIE_WAVE, lane = threadIdx.x % TIE_WAVE;
   const int p = lane & (DELTA_PARTS - 1), c = lane / DELTA_PARTS;
   const int first_col = (blockIdx.y * DELTA_WAVES + wave) * DELTA_COLS;
   const int col = first_col + c;
-  const bool live = col < e;
-  const int t0 = query_start[s], t1 = query_start[s + 1];
+  const int columns = mode.columns;
+  const bool live = col < columns;
+  int t0, t1, holder;
+  if (mode.items) {
+    t0 = mode.items[3 * item + 1], t1 = mode.items[3 * item + 2], holder = item;
+  } else {
+    t0 = query_start[item], t1 = query_start[item + 1], holder = state_slots[item];
+  }
   if (t0 >= t1) return;                               // the whole workgroup
-  float* sp = state + ((static_cast<size_t>(state_slots[s]) * H + head) * d) * e + col;
+  float* sp = state + ((static_cast<size_t>(holder) * H + head) * d) * columns + col;
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = p * R + r;
-    S[r] = (live && i < d) ? sp[static_cast<size_t>(i) * e] : 0.f;
+    if (mode.init) S[r] = (live && col - e == i) ? 1.f : 0.f;
+    else S[r] = (live && i < d) ? sp[static_cast<size_t>(i) * columns] : 0.f;
   }
   DeltaRowPlan pl;
   pl.q_at = kv * d;
@@ -315,6 +336,7 @@ __global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
   pl.first_col = first_col;
   pl.d = d, pl.e = e, pl.t1 = t1, pl.row = row;
   float* vb = vbs[wave];
+  const bool writes = mode.outputs && p == 0 && col < e;
   float stage[PER][W], stage_vb[VB];
   delta_fetch<DP, NT, W, PER>(tok, pl, t0, stage);
   delta_fetch_values<NT, VB>(tok, pl, t0, lane, stage_vb);
@@ -360,7 +382,7 @@ __global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
       for (int j = 0; j < count; ++j) {
         read(j, ka, qa, ga);
         const float sum = delta_token<R>(S, ka, qa, ga, vb[j * (DELTA_COLS + 1) + c], vb[j * (DELTA_COLS + 1) + DELTA_COLS]);
-        if (p == 0 && live) o[static_cast<size_t>(j) * out_row] = sum;
+        if (writes) o[static_cast<size_t>(j) * out_row] = sum;
       }
       continue;
     }
@@ -368,41 +390,140 @@ __global__ __launch_bounds__(DELTA_THREADS) void gated_delta_scan_kernel(
     for (int j = 0; j < count; j += 2) {
       if (j + 1 < count) read(j + 1, kb, qb, gb);
       const float first = delta_token<R>(S, ka, qa, ga, vb[j * (DELTA_COLS + 1) + c], vb[j * (DELTA_COLS + 1) + DELTA_COLS]);
-      if (p == 0 && live) o[static_cast<size_t>(j) * out_row] = first;
+      if (writes) o[static_cast<size_t>(j) * out_row] = first;
       if (j + 1 < count) {
         if (j + 2 < count) read(j + 2, ka, qa, ga);
         const float second = delta_token<R>(S, kb, qb, gb, vb[(j + 1) * (DELTA_COLS + 1) + c],
                                             vb[(j + 1) * (DELTA_COLS + 1) + DELTA_COLS]);
-        if (p == 0 && live) o[static_cast<size_t>(j + 1) * out_row] = second;
+        if (writes) o[static_cast<size_t>(j + 1) * out_row] = second;
       }
     }
   }
+  if (!mode.store) return;
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = p * R + r;
-    if (live && i < d) sp[static_cast<size_t>(i) * e] = S[r];
+    if (live && i < d) sp[static_cast<size_t>(i) * columns] = S[r];
   }
 }
 
+// The chunks' states in order: `ends` [count][H][d][e + d] holds what every chunk makes of a zero state (columns
+// below e) and its transition P (columns from e on). A workgroup owns COMBINE_COLS columns of a (sequence, head):
+// it leaves every chunk the state before its first token (`starts` [count][H][d][e]) and the slot the state behind
+// the last one, S <- P S + L chunk after chunk. A thread has a row (two where d > 128) and four columns; the state
+// lies in LDS, and P passes through LDS `jt` columns at a time (rows jt + 1 words apart: the rows of a wave meet
+// different banks), the next tile on its way into registers meanwhile.
+#define COMBINE_COLS 8
+#define COMBINE_THREADS 256
+#define COMBINE_TILE 8192          // elements of P in LDS at a time
+#define COMBINE_PER (COMBINE_TILE / COMBINE_THREADS)
+
+__global__ __launch_bounds__(COMBINE_THREADS) void gated_delta_combine_kernel(
+    const float* __restrict__ ends, float* __restrict__ starts, float* __restrict__ state,
+    const int* __restrict__ first_chunk, const int* __restrict__ state_slots, int H, int d, int e, int jt) {
+  extern __shared__ __attribute__((aligned(16))) float sl[];       // [2][d][COMBINE_COLS], then P's tile [d][jt + 1]
+  const int s = blockIdx.x / H, head = blockIdx.x % H;
+  const int c0 = first_chunk[s], c1 = first_chunk[s + 1];
+  if (c0 >= c1) return;
+  const int col0 = blockIdx.y * COMBINE_COLS;
+  const int half = threadIdx.x & 1, col = col0 + half * 4;          // this thread's four columns
+  const int row0 = threadIdx.x >> 1;                                // its rows: row0, row0 + 128
+  float* slot = state + (static_cast<size_t>(state_slots[s]) * H + head) * d * e;
+  float* cur = sl;
+  float* nxt = sl + d * COMBINE_COLS;
+  float* pl = sl + 2 * d * COMBINE_COLS;
+  for (int i = row0; i < d; i += COMBINE_THREADS / 2)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) cur[i * COMBINE_COLS + half * 4 + x] = col + x < e ? slot[static_cast<size_t>(i) * e + col + x] : 0.f;
+  const int wide = e + d;
+  const int tiles = (d + jt - 1) / jt;
+  float ahead[COMBINE_PER];
+  // element k * COMBINE_THREADS + thread of a tile is (row, column) = (i0 + k * rows_step, jj0) where jt divides the
+  // threads; otherwise a division an element
+  const bool regular = COMBINE_THREADS % jt == 0;
+  const int i0 = threadIdx.x / jt, jj0 = threadIdx.x % jt, rows_step = COMBINE_THREADS / jt;
+  auto fetch = [&](int c, int tile) {            // tile `tile` of chunk c's P into registers
+    const float* P = ends + (static_cast<size_t>(c) * H + head) * d * wide + e + tile * jt;
+    const int width = min(jt, d - tile * jt);
+#pragma unroll
+    for (int k = 0; k < COMBINE_PER; ++k) {
+      int i = i0 + k * rows_step, jj = jj0;
+      if (!regular) i = (k * COMBINE_THREADS + threadIdx.x) / jt, jj = (k * COMBINE_THREADS + threadIdx.x) % jt;
+      ahead[k] = (i < d && jj < width) ? P[static_cast<size_t>(i) * wide + jj] : 0.f;
+    }
+  };
+  fetch(c0, 0);
+  float acc[2][4];
+  for (int c = c0; c < c1; ++c) {
+    const float* E = ends + (static_cast<size_t>(c) * H + head) * d * wide;
+    float* st = starts + (static_cast<size_t>(c) * H + head) * d * e;
+    for (int tile = 0; tile < tiles; ++tile) {
+      __syncthreads();                             // the tile before is used up; `cur` is whole
+#pragma unroll
+      for (int k = 0; k < COMBINE_PER; ++k) {
+        int i = i0 + k * rows_step, jj = jj0;
+        if (!regular) i = (k * COMBINE_THREADS + threadIdx.x) / jt, jj = (k * COMBINE_THREADS + threadIdx.x) % jt;
+        if (i < d) pl[i * (jt + 1) + jj] = ahead[k];
+      }
+      __syncthreads();
+      if (tile + 1 < tiles) fetch(c, tile + 1);
+      else if (c + 1 < c1) fetch(c + 1, 0);
+      const int width = min(jt, d - tile * jt);
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const int i = row0 + rr * (COMBINE_THREADS / 2);
+        if (i >= d) continue;
+        if (tile == 0) {
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            if (col + x < e) st[static_cast<size_t>(i) * e + col + x] = cur[i * COMBINE_COLS + half * 4 + x];
+            acc[rr][x] = col + x < e ? E[static_cast<size_t>(i) * wide + col + x] : 0.f;
+          }
+        }
+        const float* pi = pl + i * (jt + 1);
+        const float* sj = cur + tile * jt * COMBINE_COLS + half * 4;
+        for (int jj = 0; jj < width; ++jj) {
+          const float pij = pi[jj];
+          const float4 v = *reinterpret_cast<const float4*>(sj + jj * COMBINE_COLS);
+          acc[rr][0] = fmaf(pij, v.x, acc[rr][0]);
+          acc[rr][1] = fmaf(pij, v.y, acc[rr][1]);
+          acc[rr][2] = fmaf(pij, v.z, acc[rr][2]);
+          acc[rr][3] = fmaf(pij, v.w, acc[rr][3]);
+        }
+        if (tile + 1 == tiles) {
+#pragma unroll
+          for (int x = 0; x < 4; ++x) nxt[i * COMBINE_COLS + half * 4 + x] = acc[rr][x];
+        }
+      }
+    }
+    float* t = cur;
+    cur = nxt;
+    nxt = t;
+  }
+  __syncthreads();
+  for (int i = row0; i < d; i += COMBINE_THREADS / 2)
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+      if (col + x < e) slot[static_cast<size_t>(i) * e + col + x] = cur[i * COMBINE_COLS + half * 4 + x];
+}
+
 // tok: rows of delta_prepare; out: float32 [T][>= H e]; state: [slots][H][d][e].
-extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int out_row, float* state,
-                                    const int* query_start, const int* state_slots, int num_seqs, int G, int H, int d,
-                                    int e, hipStream_t stream) {
+static int launch_delta_scan(const float* tok, int row, float* out, int out_row, float* state, const int* query_start,
+                             const int* state_slots, int num_items, int G, int H, int d, int e, DeltaScanMode mode,
+                             hipStream_t stream) {
   constexpr int wg_cols = DELTA_WAVES * DELTA_COLS;
-  if (num_seqs <= 0 || G <= 0 || H <= 0 || H % G || d <= 0 || d > 256 || e <= 0 || out_row < H * e ||
-      row < 2 * G * d + H * e + H + H * d || (e + wg_cols - 1) / wg_cols > 65535)
-    return TIE_BAD_ARGUMENT;
-  const dim3 grid(num_seqs * H, (e + wg_cols - 1) / wg_cols);
+  const dim3 grid(num_items * H, (mode.columns + wg_cols - 1) / wg_cols);
+  if (grid.y > 65535) return TIE_BAD_ARGUMENT;
   // four words a load where every head's k, q and g start at a multiple of four words of an aligned row
   const bool wide = d % 4 == 0 && (H * e) % 4 == 0 && row % 4 == 0 && reinterpret_cast<uintptr_t>(tok) % 16 == 0;
 #define SCAN(R)                                                                                                    \
   do {                                                                                                             \
     if (wide)                                                                                                      \
       gated_delta_scan_kernel<R, 4><<<grid, DELTA_THREADS, 0, stream>>>(tok, row, out, out_row, state, query_start, \
-                                                                        state_slots, G, H, d, e);                   \
+                                                                        state_slots, G, H, d, e, mode);             \
     else                                                                                                           \
       gated_delta_scan_kernel<R, 1><<<grid, DELTA_THREADS, 0, stream>>>(tok, row, out, out_row, state, query_start, \
-                                                                        state_slots, G, H, d, e);                   \
+                                                                        state_slots, G, H, d, e, mode);             \
   } while (0)
   if (d <= 32) SCAN(4);
   else if (d <= 64) SCAN(8);
@@ -410,6 +531,43 @@ extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int o
   else SCAN(32);
 #undef SCAN
   return tie_launch_status();
+}
+
+extern "C" int tie_gated_delta_scan(const float* tok, int row, float* out, int out_row, float* state,
+                                    const int* query_start, const int* state_slots, int num_seqs, int G, int H, int d,
+                                    int e, hipStream_t stream) {
+  if (num_seqs <= 0 || G <= 0 || H <= 0 || H % G || d <= 0 || d > 256 || e <= 0 || out_row < H * e ||
+      row < 2 * G * d + H * e + H + H * d)
+    return TIE_BAD_ARGUMENT;
+  return launch_delta_scan(tok, row, out, out_row, state, query_start, state_slots, num_seqs, G, H, d, e,
+                           DeltaScanMode{nullptr, e, 0, 1, 1}, stream);
+}
+
+// The same over chunks, in three launches: every chunk from a zero state with its transition beside it (`ends`
+// [count][H][d][e + d]), the chunks' states combined in order (`starts` [count][H][d][e]; the slots receive the
+// final states), every chunk again from its true start with outputs. items: [count][3] (sequence, first row, end
+// row), in the order of the sequences' rows; first_chunk: [num_seqs + 1].
+extern "C" int tie_gated_delta_scan_chunked(const float* tok, int row, float* out, int out_row, float* state,
+                                            const int* state_slots, int num_seqs, const int* items,
+                                            const int* first_chunk, int count, float* ends, float* starts, int G,
+                                            int H, int d, int e, hipStream_t stream) {
+  if (num_seqs <= 0 || count <= 0 || G <= 0 || H <= 0 || H % G || d <= 0 || d > 256 || e <= 0 || out_row < H * e ||
+      row < 2 * G * d + H * e + H + H * d || !items || !first_chunk || !ends || !starts)
+    return TIE_BAD_ARGUMENT;
+  int rc = launch_delta_scan(tok, row, out, out_row, ends, nullptr, nullptr, count, G, H, d, e,
+                             DeltaScanMode{items, e + d, 1, 1, 0}, stream);
+  if (rc != TIE_OK) return rc;
+  const dim3 grid(num_seqs * H, (e + COMBINE_COLS - 1) / COMBINE_COLS);
+  if (grid.y > 65535) return TIE_BAD_ARGUMENT;
+  int jt = COMBINE_TILE / d / 4 * 4;           // d <= 256: at least 32
+  if (jt > d) jt = d;
+  const size_t lds = (2 * static_cast<size_t>(d) * COMBINE_COLS + static_cast<size_t>(d) * (jt + 1)) * sizeof(float);
+  gated_delta_combine_kernel<<<grid, COMBINE_THREADS, lds, stream>>>(ends, starts, state, first_chunk, state_slots, H,
+                                                                     d, e, jt);
+  rc = tie_launch_status();
+  if (rc != TIE_OK) return rc;
+  return launch_delta_scan(tok, row, out, out_row, starts, nullptr, nullptr, count, G, H, d, e,
+                           DeltaScanMode{items, e, 0, 0, 1}, stream);
 }
 
 // ---------------------------------------------------------------- the norm of the heads' outputs, gated

@@ -148,6 +148,8 @@ _SIGNATURES = {
                               _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void],
         "tie_gated_delta_scan": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_void],
+        "tie_gated_delta_scan_chunked": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_void,
+                                         _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_void],
         "tie_grouped_gated_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int,
                                        _c_int, _c_int, _c_void],
     },
@@ -2049,11 +2051,23 @@ def delta_prepare(u: torch.Tensor, weight: torch.Tensor, taps: int, state: Optio
           out.stride(0), _stream())
 
 
+DELTA_CHUNK_ROWS = 256                 # rows of a chunk of the gated delta rule's chunked walk
+DELTA_CHUNKS_FROM = 1024               # a step's longest portion from which the rule runs in chunks (three launches)
+DELTA_CHUNK_SCRATCH_MAX = 1 << 30      # bytes of chunk states above which a step walks its sequences whole
+
+
 def gated_delta_scan(tok: torch.Tensor, out: torch.Tensor, state: torch.Tensor, batch, kv_heads: int, heads: int,
-                     key_dim: int, value_dim: int) -> None:
+                     key_dim: int, value_dim: int, chunks: Optional[ScanChunks] = None, scratch=None) -> None:
     """The gated delta rule, token by token through each sequence's state ``[slots, H, d, e]`` (float32):
     ``S <- decay * S`` row by row; ``u = beta * (v - S^T k)``; ``S <- S + k u^T``; ``o = S^T q``. ``tok``: the rows of
-    ``delta_prepare``; ``out`` float32 ``[T, H e]``."""
+    ``delta_prepare``; ``out`` float32 ``[T, H e]``.
+
+    With ``chunks`` (``scan_chunks``; ``scratch(name, shape, dtype)`` hands out the memory for the chunks' states)
+    the rows run chunk beside chunk in three launches. A token's step is linear in the state,
+    ``S_t = (I - beta k k^T) diag(decay) S_(t-1) + beta k v^T``, so a chunk is ``S_end = P S_start + L``: every chunk
+    walks from a zero state with ``d`` more columns that start as the identity and take no values (they end as
+    ``P``), the chunks' states are combined in order, and every chunk walks again from its true start, with
+    outputs. The same values up to rounding."""
     G, H, d, e = kv_heads, heads, key_dim, value_dim
     T = tok.shape[0]
     _f32(tok, "delta rule rows", (T, 2 * G * d + H * e + H + H * d))
@@ -2063,6 +2077,14 @@ def gated_delta_scan(tok: torch.Tensor, out: torch.Tensor, state: torch.Tensor, 
         raise InvalidArgument(f"a state {list(state.shape)} does not fit {H} heads of {d} x {e} (keys up to "
                               f"{DELTA_RULE_MAX_DIM}, {G} key heads)")
     if batch.num_seqs == 0:
+        return
+    if chunks is not None and chunks.count * H * d * (e + d) * 4 <= DELTA_CHUNK_SCRATCH_MAX:
+        ends = scratch("delta_rule.chunk_ends", (chunks.count, H, d, e + d), torch.float32)
+        starts = scratch("delta_rule.chunk_starts", (chunks.count, H, d, e), torch.float32)
+        _call(_lib("delta_rule").tie_gated_delta_scan_chunked, "gated_delta_scan_chunked", tok.data_ptr(),
+              tok.stride(0), out.data_ptr(), out.stride(0), state.data_ptr(), batch.state_slots.data_ptr(),
+              batch.num_seqs, chunks.items.data_ptr(), chunks.first_item.data_ptr(), chunks.count, ends.data_ptr(),
+              starts.data_ptr(), G, H, d, e, _stream())
         return
     _call(_lib("delta_rule").tie_gated_delta_scan, "gated_delta_scan", tok.data_ptr(), tok.stride(0), out.data_ptr(),
           out.stride(0), state.data_ptr(), batch.query_start.data_ptr(), batch.state_slots.data_ptr(), batch.num_seqs,

@@ -259,8 +259,11 @@ class GatedDeltaRule(Mixer):
         if conv_state is not None and state.writes:
             kernels.conv_state_update(proj, self.taps, conv_state, ctx.batch, self.channels)
         o = ctx.scratch("delta_rule.o", (T, self.v_width), torch.float32)
+        chunks = None
+        if max(ctx.batch.host_new_tokens) >= kernels.DELTA_CHUNKS_FROM:      # such steps are never recorded
+            chunks = kernels.scan_chunks(ctx.batch, ctx.device, rows=kernels.DELTA_CHUNK_ROWS)
         kernels.gated_delta_scan(tok, o, state.state, ctx.batch, self.kv_heads, self.heads, self.key_dim,
-                                 self.value_dim)
+                                 self.value_dim, chunks=chunks, scratch=ctx.scratch)
         gated = ctx.scratch("delta_rule.gated", (T, self.v_width))
         kernels.grouped_gated_rms_norm(o, self.norm_weight, self.eps, second[:, self.decay_width:], gated, self.heads)
         return _finish(ctx, self.out, gated, residual, "delta_rule.result")
