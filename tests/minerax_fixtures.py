@@ -5,7 +5,7 @@ A has two residual streams, latent attention with three heads whose cached head 
 with two convolution taps and capped scores beside a delta rule with grouped query/key heads, and layers without a
 feed-forward. B has one plain residual (no streams), twenty latent heads (more than the matrix-core decode kernel
 takes), a rotation of whole heads on the left, four taps, no cap, ungrouped delta-rule heads whose keys are wider
-than their values. C has one stream, sizes in no step of 8, a window longer than any request, convolutions of one
+than their values. C has one stream, sizes in no step of 8, latent attention without a window, convolutions of one
 tap (no state), no stretched frequencies, no rotation on the left at all. D has four streams and only side-by-side
 layers, two of them (their states share groups), and keys of 64. E is latent attention alone with a window of one
 position (a token sees itself and the sink).
@@ -68,7 +68,7 @@ B = {
 C = {
     "architecture": "Minerax", "vocab": 333, "width": 100, "norm": {"eps": 1e-4}, "streams": 1,
     "layers": [
-        {"type": "latent_attention", "mixer": _latent(5, 10, 6, 7, 13, 0.3, 200, 30.0),
+        {"type": "latent_attention", "mixer": _latent(5, 10, 6, 7, 13, 0.3, None, 30.0),
          "mlp": {"kind": "dense", "ff": 50}},
         {"type": "parallel",
          "mixer": {"left": {"heads": 3, "kv_heads": 3, "dim": 12, "vdim": 12, "conv": 1, "scale": 0.28},

@@ -46,7 +46,7 @@ def step_batch(counts, slots):
 
 
 # ------------------------------------------------------------------------------------------- kernels alone
-@pytest.mark.parametrize("n", [20, 64, 100, 320, 2048, 5000])
+@pytest.mark.parametrize("n", [20, 64, 100, 384, 2048, 5000])
 def test_layer_norm_kernel(n):
     from tie_amd import kernels
 
@@ -64,7 +64,7 @@ def test_layer_norm_kernel(n):
     close(out, plain.layer_norm(half.cpu().to(F64), w.cpu().to(F64), 1e-5), 2e-6, "layer norm of bfloat16 rows")
 
 
-@pytest.mark.parametrize("S,n,planes", [(1, 48, 0), (2, 64, 1), (3, 320, 0), (4, 100, 3), (8, 1000, 2)])
+@pytest.mark.parametrize("S,n,planes", [(1, 48, 0), (2, 64, 1), (3, 352, 0), (4, 100, 3), (8, 1000, 2), (4, 4100, 2), (2, 9000, 1)])
 def test_hyper_connection_kernel(S, n, planes):
     from tie_amd import kernels
 
