@@ -4,6 +4,7 @@
     python bench.py --shape 32b                 the same measurements at the Qwen3-32B sizes
     python bench.py --sweep [--shape 32b]       decode at contexts 4096 / 16384 / 32768 x batch 1 / 8 / 32, a line a point
     python bench.py --workload stress           64 requests through the scheduler at the Qwen3-1.7B sizes
+    python bench.py --workload minerax          another design beside Qwen3 at equal sizes (also duzozen, topapel): prefill, decode
 
 Prints ONE JSON line. A "step" is one decode step of the engine (schedule, build the batch, run
 the model, sample greedily) at the default batch of 8 with every sequence near the benchmark
