@@ -50,8 +50,11 @@ __global__ void conv_qkv_kernel(const float* __restrict__ u, int row, const floa
   const int start = query_start[s];
   const int C = nq + nk + nv;
   const float* hist = state + static_cast<size_t>(state_slots[s]) * (taps - 1) * C;
+  // three workgroups a row: q, k and v each on their own (a norm runs over one of them)
+  const int lo = blockIdx.y == 0 ? 0 : (blockIdx.y == 1 ? nq : nq + nk);
+  const int hi = blockIdx.y == 0 ? nq : (blockIdx.y == 1 ? nq + nk : C);
   float sq = 0.f, sk = 0.f;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int c = lo + threadIdx.x; c < hi; c += blockDim.x) {
     const float y = taps > 1 ? conv_at(u, row, w, hist, taps, C, t, start, c)
                              : w[c] * u[static_cast<size_t>(t) * row + c];
     vals[c] = y;
@@ -59,11 +62,11 @@ __global__ void conv_qkv_kernel(const float* __restrict__ u, int row, const floa
     else if (c < nq + nk) sk = fmaf(y, y, sk);
   }
   float iq = 1.f, ik = 1.f;
-  if (wq) iq = 1.0f / sqrtf(block_sum(sq, scratch) / count_q + eps);
-  if (wk) ik = 1.0f / sqrtf(block_sum(sk, scratch) / count_k + eps);
+  if (wq && blockIdx.y == 0) iq = 1.0f / sqrtf(block_sum(sq, scratch) / count_q + eps);
+  if (wk && blockIdx.y == 1) ik = 1.0f / sqrtf(block_sum(sk, scratch) / count_k + eps);
   __syncthreads();
   float* o = out + static_cast<size_t>(t) * out_row;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int c = lo + threadIdx.x; c < hi; c += blockDim.x) {
     float y = vals[c];
     if (c < nq) { if (wq) y = (y * iq) * wq[c]; }
     else if (c < nq + nk) { if (wk) y = (y * ik) * wk[c - nq]; }
@@ -81,7 +84,7 @@ extern "C" int tie_conv_qkv(const float* u, int row, const float* w, int taps, c
     return TIE_BAD_ARGUMENT;
   // few channels a thread: every one waits for its loads, and a decode step brings few rows
   const int threads = C >= 2048 ? 1024 : (C >= 1024 ? 512 : (C >= 512 ? 256 : 128));
-  conv_qkv_kernel<<<T, threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
+  conv_qkv_kernel<<<dim3(T, 3), threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
       u, row, w, taps, state, state_slots, seq_of_row, query_start, nq, nk, nv, wq, wk, count_q, count_k, eps, out,
       out_row);
   return tie_launch_status();
@@ -139,13 +142,25 @@ __global__ void delta_prepare_kernel(const float* __restrict__ u, int row, const
   const int start = query_start[s];
   const int C = 2 * G * d + H * e;
   const float* hist = state + static_cast<size_t>(state_slots[s]) * (taps - 1) * C;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  float* o = out + static_cast<size_t>(t) * out_row;
+  // three workgroups a row: q and k with their unit norms, v, and beta with the decays
+  if (blockIdx.y == 2) {
+    const float* b = u + static_cast<size_t>(t) * row + C;
+    for (int h = threadIdx.x; h < H; h += blockDim.x) o[C + H * d + h] = sigmoid_f(b[h]);
+    const float* ar = a + static_cast<size_t>(t) * a_row;
+    for (int c = threadIdx.x; c < H * d; c += blockDim.x)
+      o[C + c] = expf(-expf(A_log[c / d]) * softplus_f(ar[c] + dt_bias[c]));
+    return;
+  }
+  const int lo = blockIdx.y == 0 ? 0 : 2 * G * d, hi = blockIdx.y == 0 ? 2 * G * d : C;
+  for (int c = lo + threadIdx.x; c < hi; c += blockDim.x) {
     const float y = taps > 1 ? conv_at(u, row, w, hist, taps, C, t, start, c)
                              : w[c] * u[static_cast<size_t>(t) * row + c];
-    vals[c] = silu_f(y);
+    if (blockIdx.y == 0) vals[c] = silu_f(y);
+    else o[c] = silu_f(y);
   }
+  if (blockIdx.y == 1) return;
   __syncthreads();
-  float* o = out + static_cast<size_t>(t) * out_row;
   const int lane = threadIdx.x & (TIE_WAVE - 1), wave = threadIdx.x / TIE_WAVE, waves = blockDim.x / TIE_WAVE;
   const float q_scale = 1.0f / sqrtf(static_cast<float>(d));
   for (int head = wave; head < 2 * G; head += waves) {      // q heads, then k heads
@@ -156,12 +171,6 @@ __global__ void delta_prepare_kernel(const float* __restrict__ u, int row, const
     const float f = head < G ? inv * q_scale : inv;
     for (int i = lane; i < d; i += TIE_WAVE) o[head * d + i] = x[i] * f;
   }
-  for (int c = 2 * G * d + threadIdx.x; c < C; c += blockDim.x) o[c] = vals[c];
-  const float* b = u + static_cast<size_t>(t) * row + C;
-  for (int h = threadIdx.x; h < H; h += blockDim.x) o[C + H * d + h] = sigmoid_f(b[h]);
-  const float* ar = a + static_cast<size_t>(t) * a_row;
-  for (int c = threadIdx.x; c < H * d; c += blockDim.x)
-    o[C + c] = expf(-expf(A_log[c / d]) * softplus_f(ar[c] + dt_bias[c]));
 }
 
 extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int taps, const float* state,
@@ -173,7 +182,7 @@ extern "C" int tie_delta_prepare(const float* u, int row, const float* w, int ta
       out_row < C + H + H * d || a_row < H * d || static_cast<size_t>(C) * 4 > 65536 || (taps > 1 && !state))
     return TIE_BAD_ARGUMENT;
   const int threads = C >= 2048 ? 1024 : (C >= 1024 ? 512 : 256);
-  delta_prepare_kernel<<<T, threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
+  delta_prepare_kernel<<<dim3(T, 3), threads, static_cast<size_t>(C) * sizeof(float), stream>>>(
       u, row, w, taps, state, state_slots, seq_of_row, query_start, a, a_row, A_log, dt_bias, G, H, d, e, out,
       out_row);
   return tie_launch_status();

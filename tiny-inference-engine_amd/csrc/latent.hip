@@ -39,13 +39,20 @@ __global__ void latent_prepare_kernel(const float* __restrict__ proj, int row, c
     return first ? x[i] * c - x[partner] * s : x[i] * c + x[partner] * s;
   };
   const int qw = d + r;
-  for (int i = threadIdx.x; i < H * d; i += blockDim.x) {
-    const int h = i / d, j = i % d;
-    store_from_float(qn + t * (static_cast<size_t>(H) * d) + i, p[h * qw + j]);
+  // three workgroups a row, each with one part of the work: none waits for another's loads
+  if (blockIdx.y == 0) {
+    for (int i = threadIdx.x; i < H * d; i += blockDim.x) {
+      const int h = i / d, j = i % d;
+      store_from_float(qn + t * (static_cast<size_t>(H) * d) + i, p[h * qw + j]);
+    }
+    return;
   }
-  for (int i = threadIdx.x; i < H * (D - kr); i += blockDim.x) {
-    const int h = i / (D - kr), j = i % (D - kr);
-    store_from_float(qa + (t * H + h) * D + kr + j, j < r ? rotated(p + h * qw + d, j) : 0.f);
+  if (blockIdx.y == 1) {
+    for (int i = threadIdx.x; i < H * (D - kr); i += blockDim.x) {
+      const int h = i / (D - kr), j = i % (D - kr);
+      store_from_float(qa + (t * H + h) * D + kr + j, j < r ? rotated(p + h * qw + d, j) : 0.f);
+    }
+    return;
   }
   if (!write_kv) return;
   const float* c_raw = p + H * qw;
@@ -75,7 +82,7 @@ extern "C" int tie_latent_prepare(const float* proj, int row, const float* w_c, 
   if (write_kv && (!slots || !k_cache || !v_cache)) return TIE_BAD_ARGUMENT;
   const int threads = 256;
 #define LP(TA, TC)                                                                                                   \
-  latent_prepare_kernel<TA, TC><<<T, threads, 0, stream>>>(proj, row, w_c, eps, angles, rdims, interleaved, slots,   \
+  latent_prepare_kernel<TA, TC><<<dim3(T, 3), threads, 0, stream>>>(proj, row, w_c, eps, angles, rdims, interleaved, slots,   \
                                                            static_cast<TC*>(k_cache), static_cast<TC*>(v_cache),      \
                                                            block_size, write_kv, static_cast<TA*>(qn),                \
                                                            static_cast<TA*>(qa), H, d, r, kr, D)
