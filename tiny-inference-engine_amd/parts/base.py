@@ -179,6 +179,7 @@ class StepContext:
         self.notes: Dict[Any, Any] = {}   # per-step memo shared by parts (e.g. one plan for all layers)
         self._owed = None                  # (target, planes): target += planes[0] + planes[1] + ... is still to be done
         self._pending = None               # (target, linear, x): target += x @ linear.weight^T is still to be launched
+        self._late = None                  # (key, run, payload): a block's last pass, left for the next block to merge
         self._row_scales: Dict[int, Any] = {}   # address of rows that lack their norm's 1 / rms -> kernels.RowScale
 
     @property
@@ -211,6 +212,20 @@ class StepContext:
             return linear, x
         return None
 
+    # A block's last pass over the residual may be left for the block behind it, which merges it into its own first
+    # pass (take_late with the same key); whoever needs the residual before that calls settle(), which runs it.
+    def leave_late(self, key, run, payload) -> None:
+        self.settle()
+        self._late = (key, run, payload)
+
+    def take_late(self, key):
+        """The payload of a pass left under ``key`` (the caller now does that work itself), or None."""
+        if self._late is None or self._late[0] != key:
+            return None
+        payload = self._late[2]
+        self._late = None
+        return payload
+
     def launch_pending(self) -> None:
         """Launches a product left pending the ordinary way (it may leave planes of partial sums owed in turn)."""
         if self._pending is not None:
@@ -241,6 +256,10 @@ class StepContext:
         return None
 
     def settle(self) -> None:
+        if self._late is not None:
+            _, run, payload = self._late
+            self._late = None
+            run(payload)
         self.launch_pending()
         if self._owed is not None:
             from .. import kernels

@@ -181,6 +181,8 @@ class HyperConnectionsBlock(Block):
 
     def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
         T = x.shape[0]
+        # the layer before may have left its last write for this layer's first pass (same streams, same rows)
+        left = ctx.take_late(("hyper.write", self.streams, T, self.hidden))
         ctx.settle()
         streams = ctx.scratch("hyper.streams", (self.streams, T, self.hidden), torch.float32)
         subs = [(s, part, layer.norms[n]) for s, n, part in
@@ -188,7 +190,12 @@ class HyperConnectionsBlock(Block):
         fresh = ctx.notes.get("hyper.streams") is None     # the first layer of the step: the streams are x
         ctx.notes["hyper.streams"] = streams
         read, h, u = self._read(ctx, subs[0][0], subs[0][2], T)
-        kernels.hyper_connection(streams, x, from_x=fresh, read=read)
+        if left is not None and not fresh:
+            kernels.hyper_connection(streams, x, write=left, read=read)       # x is not needed in between
+        else:
+            if left is not None:
+                kernels.hyper_connection(streams, x, fold=True, write=left)
+            kernels.hyper_connection(streams, x, from_x=fresh, read=read)
         for i, (sub, part, norm) in enumerate(subs):
             if h is None:
                 h = norm.forward(ctx, u)
@@ -202,4 +209,11 @@ class HyperConnectionsBlock(Block):
             if not last:
                 read, h, u = self._read(ctx, subs[i + 1][0], subs[i + 1][2], T)
             _, out_w, mix = self.weights[sub]
-            kernels.hyper_connection(streams, x, fold=last, write=(y, mix, out_w), read=read)
+            if last:
+                # left for the next layer's first pass; settle() (the model's end, a hook, another kind of block)
+                # runs it with the fold of the streams' sum into x
+                ctx.leave_late(("hyper.write", self.streams, T, self.hidden),
+                               lambda write: kernels.hyper_connection(streams, x, fold=True, write=write),
+                               (y, mix, out_w))
+            else:
+                kernels.hyper_connection(streams, x, write=(y, mix, out_w), read=read)
