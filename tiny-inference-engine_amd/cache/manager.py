@@ -277,7 +277,8 @@ class CacheManager:
         """Gives back pages of windowed groups that no later query can read; returns how many.
 
         The next query sits at position ``computed`` or later and reads keys from
-        ``computed - window + 1`` on (or from the start of its chunk), so pages wholly below that are free to go.
+        ``computed - window + 1`` on (or from the start of its chunk), so pages wholly below that are free to go,
+        except those of the first positions that a window keeps (``PagedKV.keep_first``).
         Their table entries stay (as FREED) so that positions keep their index.
         """
         freed = 0
@@ -290,7 +291,8 @@ class CacheManager:
             first_page = need.first_needed(computed) // self.block_size
             table = req.tables[g]
             first_page = min(first_page, len(table))
-            for i in range(req.trimmed[g], first_page):
+            kept = self.blocks_for(need.keep_first)          # pages of the first positions every query reads
+            for i in range(max(req.trimmed[g], kept), first_page):
                 if table[i] != FREED:
                     pool.release(table[i])
                     table[i] = FREED

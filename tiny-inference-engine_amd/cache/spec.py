@@ -29,12 +29,15 @@ class PagedKV:
     given back while the request still runs. ``chunk`` = n means a query at position p
     reads the keys of its own chunk, from p - p % n on (chunks of n positions counted from 0):
     pages wholly before the chunk of the next query can go as well. At most one of the two.
+    ``keep_first`` = f (with a window only) means every query also reads the keys of positions below f, at their
+    true positions, however far back they lie: the pages that hold them stay with the request to its end.
     """
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     chunk: Optional[int] = None
+    keep_first: int = 0
 
     def __post_init__(self):
         if self.num_kv_heads <= 0 or self.head_dim <= 0:
@@ -45,11 +48,16 @@ class PagedKV:
             raise InvalidArgument(f"an attention chunk must be positive, got {self.chunk}")
         if self.window is not None and self.chunk is not None:
             raise InvalidArgument("a paged cache has a window or chunks, not both")
+        if self.keep_first < 0 or (self.keep_first and self.window is None):
+            raise InvalidArgument(f"first positions are kept ({self.keep_first}) beside a window only, and not a "
+                                  f"negative number of them")
 
     @property
     def reach(self) -> Optional[int]:
         """The most positions a query reads (None: all of them): what a request must hold at a time."""
-        return self.window if self.window is not None else self.chunk
+        if self.window is not None:
+            return self.window + self.keep_first
+        return self.chunk
 
     def first_needed(self, position: int) -> int:
         """The first key any query at ``position`` or later reads."""

@@ -8,7 +8,9 @@
 // pos - window + 1 (a sliding window) or pos - pos % chunk (causal chunks counted from
 // position 0 of the sequence); query head h reads KV head h / (H / KVH). With sinks,
 // head h's softmax has exp(sinks[h]) as one more term of its denominator: a key that
-// has no value and whose score is not scaled. Scores are
+// has no value and whose score is not scaled. With keep > 0 (beside a window) the keys of positions
+// below keep are read as well, at their true positions, however far back they lie: the walk takes the
+// kept keys that the window does not hold first (chunks from position 0), then the window's. Scores are
 // scale * (q . k); the softmax is the online form over chunks of 256 keys, with
 // running maximum, sum and accumulator in float32
 // (reference: src/backend/cpu/cpu_backend.cpp:261-319, which walks key by key).
@@ -33,7 +35,7 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache, TO* __restrict__ out,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_of_row, int H, int KVH, int Dh,
-    int block_size, int max_blocks, float scale, float softcap, int window, int chunk,
+    int block_size, int max_blocks, float scale, float softcap, int window, int chunk, int keep,
     const float* __restrict__ sinks) {
   extern __shared__ float smem[];
   const int groups = Dh >= AT ? 1 : AT / Dh;          // key groups that accumulate P.V side by side
@@ -62,10 +64,16 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
   const bool active = wide ? (tid < Dh) : (tid < groups * Dh);
 
   float m = -INFINITY, l = 0.f, acc0 = 0.f, acc1 = 0.f;
-  for (int base = start; base <= pos; base += AT) {
+  // Two ranges of keys: the kept first positions the window has left behind, [0, min(keep, start)), then
+  // [start, pos]. Both depend on the position alone.
+  const int kept_end = min(keep, start);
+  for (int range = kept_end > 0 ? 0 : 1; range < 2; ++range) {
+  const int range_begin = range == 0 ? 0 : start;
+  const int range_last = range == 0 ? kept_end - 1 : pos;
+  for (int base = range_begin; base <= range_last; base += AT) {
     const int j = base + tid;
     float sc = -INFINITY;
-    if (j <= pos) {
+    if (j <= range_last) {
       const size_t off =
           ((static_cast<size_t>(table[j / block_size]) * KVH + kvh) * block_size + j % block_size) * Dh;
       sc = scale * dot_row(q_s, k_cache + off, Dh);
@@ -74,14 +82,14 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
     const float cmax = block_max(sc, scratch);
     const float m_new = fmaxf(m, cmax);
     const float corr = expf(m - m_new);               // exp(-inf) = 0 on the first chunk
-    const float p = (j <= pos) ? expf(sc - m_new) : 0.f;
+    const float p = (j <= range_last) ? expf(sc - m_new) : 0.f;
     p_s[tid] = p;
     const float csum = block_sum(p, scratch);         // its barriers also publish p_s
     l = l * corr + csum;
     acc0 *= corr;
     acc1 *= corr;
     m = m_new;
-    const int nkeys = min(AT, pos - base + 1);
+    const int nkeys = min(AT, range_last - base + 1);
     if (active) {
       for (int jj = g; jj < nkeys; jj += groups) {
         const int j2 = base + jj;
@@ -94,6 +102,7 @@ __global__ __launch_bounds__(AT) void paged_attention_generic_kernel(
       }
     }
     __syncthreads();                                  // p_s is rewritten by the next chunk
+  }
   }
 
   if (sinks != nullptr) {   // the sink joins the denominator under the same running maximum
@@ -123,10 +132,10 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
                                            int cache_dtype, void* out, int out_dtype, const int* query_start,
                                            const int* context_lens, const int* block_tables,
                                            const int* seq_of_row, int T, int H, int KVH, int Dh, int block_size,
-                                           int max_blocks, float scale, float softcap, int window, int chunk, const float* sinks,
-                                           hipStream_t stream) {
+                                           int max_blocks, float scale, float softcap, int window, int chunk, int keep,
+                                           const float* sinks, hipStream_t stream) {
   if (T <= 0 || T > 65535 || H <= 0 || KVH <= 0 || H % KVH != 0 || Dh <= 0 || Dh > 2 * AT || block_size <= 0 ||
-      max_blocks <= 0 || (window > 0 && chunk > 0))
+      max_blocks <= 0 || (window > 0 && chunk > 0) || keep < 0 || (keep > 0 && window <= 0))
     return TIE_BAD_ARGUMENT;
   const int groups = Dh >= AT ? 1 : AT / Dh;
   const size_t shared = sizeof(float) * (Dh + AT + groups * Dh + 16);
@@ -135,7 +144,7 @@ extern "C" int tie_paged_attention_generic(const void* q, int q_dtype, const voi
   paged_attention_generic_kernel<TQ, TC, TO><<<grid, AT, shared, stream>>>(                                  \
       static_cast<const TQ*>(q), static_cast<const TC*>(k_cache), static_cast<const TC*>(v_cache),          \
       static_cast<TO*>(out), query_start, context_lens, block_tables, seq_of_row, H, KVH, Dh, block_size,   \
-      max_blocks, scale, softcap, window, chunk, sinks)
+      max_blocks, scale, softcap, window, chunk, keep, sinks)
   if (q_dtype == TIE_F32 && cache_dtype == TIE_F32 && out_dtype == TIE_F32) LAUNCH(float, float, float);
   else if (q_dtype == TIE_BF16 && cache_dtype == TIE_BF16 && out_dtype == TIE_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (q_dtype == TIE_F32 && cache_dtype == TIE_BF16 && out_dtype == TIE_F32) LAUNCH(float, bf16_t, float);

@@ -10,7 +10,9 @@
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // ---------------------------------------------------------------- cache rows and rotated query parts
-// Row t of `proj` (float32, rows `row` apart): [q: H x (d + r) | c_raw (kr) | k_rot_raw (r) | ...].
+// Row t of `proj` (float32, rows `row` apart): [q: H x (d + r) | c_raw (kr) | k_rot_raw (r) | ...]; where the queries
+// come from a product of their own (queries made from a normed latent), `lat` (rows `lat_row` apart) holds
+// [c_raw (kr) | k_rot_raw (r) | ...] instead and `proj` only the queries.
 //   c = c_raw / rms(c_raw) * w_c                         -> key cache [c | rot(k_rot_raw) | 0 ..] (D columns) and
 //                                                           value cache [c | 0 ..], transposed inside the page
 //   q_unrot[t][h] (d values)                             -> qn (activation type), [T][H d]
@@ -18,7 +20,8 @@ __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf
 // rot turns the first `rdims` of the r values by the angles of the token's position, pairs (2i, 2i + 1) where
 // `interleaved`, else (i, i + rdims / 2); angles: [T][rdims] float32, the cosines then the sines.
 template <typename TA, typename TC>
-__global__ void latent_prepare_kernel(const float* __restrict__ proj, int row, const float* __restrict__ w_c, float eps,
+__global__ void latent_prepare_kernel(const float* __restrict__ proj, int row, const float* __restrict__ lat,
+                                      int lat_row, const float* __restrict__ w_c, float eps,
                                       const float* __restrict__ angles, int rdims, int interleaved,
                                       const int* __restrict__ slots, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
                                       int block_size, int write_kv, TA* __restrict__ qn, TA* __restrict__ qa, int H,
@@ -55,7 +58,7 @@ __global__ void latent_prepare_kernel(const float* __restrict__ proj, int row, c
     return;
   }
   if (!write_kv) return;
-  const float* c_raw = p + H * qw;
+  const float* c_raw = lat != nullptr ? lat + t * lat_row : p + H * qw;
   float ss = 0.f;
   for (int i = threadIdx.x; i < kr; i += blockDim.x) ss = fmaf(c_raw[i], c_raw[i], ss);
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(kr) + eps);
@@ -72,17 +75,18 @@ __global__ void latent_prepare_kernel(const float* __restrict__ proj, int row, c
   }
 }
 
-extern "C" int tie_latent_prepare(const float* proj, int row, const float* w_c, float eps, const float* angles,
+extern "C" int tie_latent_prepare(const float* proj, int row, const float* lat, int lat_row, const float* w_c,
+                                  float eps, const float* angles,
                                   int rdims, int interleaved, const int* slots, void* k_cache, void* v_cache,
                                   int cache_dtype, int block_size, int write_kv, void* qn, void* qa, int act_dtype,
                                   int T, int H, int d, int r, int kr, int D, hipStream_t stream) {
   if (T <= 0 || H <= 0 || d <= 0 || r < 0 || kr <= 0 || D < kr + r || rdims < 0 || rdims > r || rdims % 2 ||
-      row < H * (d + r) + kr + r || block_size <= 0 || (rdims > 0 && !angles))
+      row < H * (d + r) + (lat ? 0 : kr + r) || (lat && lat_row < kr + r) || block_size <= 0 || (rdims > 0 && !angles))
     return TIE_BAD_ARGUMENT;
   if (write_kv && (!slots || !k_cache || !v_cache)) return TIE_BAD_ARGUMENT;
   const int threads = 256;
 #define LP(TA, TC)                                                                                                   \
-  latent_prepare_kernel<TA, TC><<<dim3(T, 3), threads, 0, stream>>>(proj, row, w_c, eps, angles, rdims, interleaved, slots,   \
+  latent_prepare_kernel<TA, TC><<<dim3(T, 3), threads, 0, stream>>>(proj, row, lat, lat_row, w_c, eps, angles, rdims, interleaved, slots,   \
                                                            static_cast<TC*>(k_cache), static_cast<TC*>(v_cache),      \
                                                            block_size, write_kv, static_cast<TA*>(qn),                \
                                                            static_cast<TA*>(qa), H, d, r, kr, D)
@@ -92,6 +96,32 @@ extern "C" int tie_latent_prepare(const float* proj, int row, const float* w_c, 
   else if (act_dtype == TIE_BF16 && cache_dtype == TIE_BF16) LP(bf16_t, bf16_t);
   else return TIE_BAD_ARGUMENT;
 #undef LP
+  return tie_launch_status();
+}
+
+// ---------------------------------------------------------------- an RMS norm over the first columns of wider rows
+// out[t][i] = x[t][i] / sqrt(mean_i(x[t][i]^2) + eps) * w[i] for i < n, x rows `x_row` apart (float32), out dense.
+template <typename TO>
+__global__ void rms_norm_columns_kernel(const float* __restrict__ x, int x_row, const float* __restrict__ w, float eps,
+                                        TO* __restrict__ out, int n) {
+  __shared__ float scratch[16];
+  const size_t t = blockIdx.x;
+  const float* p = x + t * x_row;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(p[i], p[i], ss);
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(n) + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) store_from_float(out + t * n + i, (p[i] * inv) * w[i]);
+}
+
+extern "C" int tie_rms_norm_columns(const float* x, int x_row, const float* w, float eps, void* out, int out_dtype,
+                                    int T, int n, hipStream_t stream) {
+  if (T <= 0 || n <= 0 || x_row < n) return TIE_BAD_ARGUMENT;
+  const int threads = n >= 1024 ? 1024 : (n >= 256 ? 256 : 64);
+  if (out_dtype == TIE_F32)
+    rms_norm_columns_kernel<float><<<T, threads, 0, stream>>>(x, x_row, w, eps, static_cast<float*>(out), n);
+  else if (out_dtype == TIE_BF16)
+    rms_norm_columns_kernel<bf16_t><<<T, threads, 0, stream>>>(x, x_row, w, eps, static_cast<bf16_t*>(out), n);
+  else return TIE_BAD_ARGUMENT;
   return tie_launch_status();
 }
 

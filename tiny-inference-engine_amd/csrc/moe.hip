@@ -1,16 +1,21 @@
 // A routed feed-forward (mixture of experts) for gfx950: the router's choice, the rows sorted by expert, and the
 // experts' two products over the sorted rows.
 //
-//   route      scores s = softmax(logits) over all experts of a row (float32); the choice looks at s + correction:
-//              experts form `groups` equal groups of neighbours, a group scores its best member, only members of the
-//              `keep` best groups stay eligible (the others count as -inf), and the `top` best of those are chosen,
-//              ties to the lower index; the weights are s at the chosen, not renormalised.
+//   route      scores s = softmax(logits) over all experts of a row, or sigmoid(logits) expert by expert (float32);
+//              the choice looks at s + correction: experts form `groups` equal groups of neighbours, a group scores
+//              its best member (or the sum of its `group_top` best), only members of the `keep` best groups stay
+//              eligible (the others count as -inf), and the `top` best of those are chosen, ties to the lower index;
+//              the weights are s at the chosen, as they are or divided by their sum (+ an eps), times a factor.
+//              `shared` further slots a row name the experts E, E + 1, ... (experts every row uses: a shared expert,
+//              cut into pieces of the routed experts' size), all with the weight sigmoid(logits[E]), one more
+//              column of the router's product.
 //   align      the T * top (row, choice) slots sorted by expert: offsets[e] .. offsets[e + 1] are the places of
 //              expert e's slots, slot_at[place] = slot, where[slot] = place (-1 for a choice >= `real`: an expert
 //              without weights, which the caller treats as it likes), and the list of row tiles (expert, first
 //              place) the products run over. Integer counters only; which place a slot gets inside its expert's
 //              range depends on timing, but no result does: a row's sums are formed the same way at every place.
-//   products   act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T)   and   parts[place] = act[place] Wd_e^T,
+//   products   act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T), or relu(x[row] Wu_e^T)^2 for experts without a
+//              gate, and   parts[place] = act[place] Wd_e^T,
 //              one workgroup a (row tile of one expert, column tile). The generic kernels multiply and add in
 //              float32 on the vector units for any sizes and float32 / bfloat16 operands (the true 32-bit path);
 //              the bfloat16 kernels run the same tiles on the matrix cores.
@@ -22,6 +27,7 @@
 #include <math.h>
 
 #define MOE_MAX_EXPERTS 1024
+#define MOE_MAX_GROUP_TOP 8     // members of a group whose scores make the group's score
 
 // ------------------------------------------------------------------ route
 // One wave a row. LDS: the scores, the choice scores, the groups' scores.
@@ -37,9 +43,11 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {   // ties: the l
   }
 }
 
-__global__ __launch_bounds__(TIE_WAVE) void moe_route_kernel(const float* __restrict__ logits,
+__global__ __launch_bounds__(TIE_WAVE) void moe_route_kernel(const float* __restrict__ logits, int row,
                                                              const float* __restrict__ correction, int E, int groups,
-                                                             int keep, int top, int* __restrict__ ids,
+                                                             int keep, int top, int sigmoid_scores, int group_top,
+                                                             int renormalize, float renorm_eps, float weight_scale,
+                                                             int shared, int* __restrict__ ids,
                                                              float* __restrict__ weights) {
   extern __shared__ float lds[];
   float* score = lds;              // [E]
@@ -47,29 +55,54 @@ __global__ __launch_bounds__(TIE_WAVE) void moe_route_kernel(const float* __rest
   float* group_score = choice + E; // [groups]
   const int lane = threadIdx.x;
   const size_t t = blockIdx.x;
-  const float* z = logits + t * E;
-  float m = -INFINITY;
-  for (int e = lane; e < E; e += TIE_WAVE) m = fmaxf(m, z[e]);
-  m = wave_max(m);
-  float sum = 0.f;
-  for (int e = lane; e < E; e += TIE_WAVE) {
-    const float p = expf(z[e] - m);
-    score[e] = p;
-    sum += p;
-  }
-  sum = wave_sum(sum);
-  for (int e = lane; e < E; e += TIE_WAVE) {
-    const float s = score[e] / sum;
-    score[e] = s;
-    choice[e] = s + (correction != nullptr ? correction[e] : 0.f);
+  const float* z = logits + t * row;
+  const int slots = top + shared;          // of a row: the chosen, then the experts every row uses
+  if (sigmoid_scores) {
+    for (int e = lane; e < E; e += TIE_WAVE) {
+      const float s = 1.0f / (1.0f + expf(-z[e]));
+      score[e] = s;
+      choice[e] = s + (correction != nullptr ? correction[e] : 0.f);
+    }
+  } else {
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += TIE_WAVE) m = fmaxf(m, z[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += TIE_WAVE) {
+      const float p = expf(z[e] - m);
+      score[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += TIE_WAVE) {
+      const float s = score[e] / sum;
+      score[e] = s;
+      choice[e] = s + (correction != nullptr ? correction[e] : 0.f);
+    }
   }
   __syncthreads();
   const int size = E / groups;
   if (groups > 1 && keep < groups) {
     for (int g = lane; g < groups; g += TIE_WAVE) {
-      float best = -INFINITY;
-      for (int j = 0; j < size; ++j) best = fmaxf(best, choice[g * size + j]);
-      group_score[g] = best;
+      // the sum of the group's `group_top` best members (1: its best), the best first; ties to the lower index
+      float total = 0.f;
+      int taken[MOE_MAX_GROUP_TOP];
+      for (int k = 0; k < group_top && k < size; ++k) {
+        float best = -INFINITY;
+        int at = -1;
+        for (int j = 0; j < size; ++j) {
+          bool used = false;
+          for (int u = 0; u < k; ++u) used = used || taken[u] == j;
+          const float v = choice[g * size + j];
+          if (!used && (at < 0 || v > best)) {
+            best = v;
+            at = j;
+          }
+        }
+        taken[k] = at;
+        total = k == 0 ? best : total + best;
+      }
+      group_score[g] = total;
     }
     __syncthreads();
     // the `keep` best groups get +inf as their mark, one at a time
@@ -104,21 +137,45 @@ __global__ __launch_bounds__(TIE_WAVE) void moe_route_kernel(const float* __rest
     wave_argmax(bv, bi);
     if (bi >= E) bi = 0;               // fewer eligible experts than `top`: a configuration's fault, not a fault here
     if (lane == 0) {
-      ids[t * top + k] = bi;
-      weights[t * top + k] = bv == -INFINITY ? 0.f : score[bi];
+      ids[t * slots + k] = bi;
+      weights[t * slots + k] = bv == -INFINITY ? 0.f : score[bi];
       choice[bi] = -INFINITY;
     }
     __syncthreads();
   }
+  if (lane == 0) {
+    float* w = weights + t * slots;
+    if (renormalize) {
+      float sum = 0.f;
+      for (int k = 0; k < top; ++k) sum += w[k];
+      sum += renorm_eps;
+      for (int k = 0; k < top; ++k) w[k] = w[k] / sum * weight_scale;
+    } else if (weight_scale != 1.0f) {
+      for (int k = 0; k < top; ++k) w[k] *= weight_scale;
+    }
+    if (shared > 0) {
+      const float g = 1.0f / (1.0f + expf(-z[E]));
+      for (int k = 0; k < shared; ++k) {
+        ids[t * slots + top + k] = E + k;
+        w[top + k] = g;
+      }
+    }
+  }
 }
 
-extern "C" int tie_moe_route(const float* logits, const float* correction, int T, int E, int groups, int keep, int top,
-                             int* ids, float* weights, hipStream_t stream) {
+// logits [T][row] float32 with row >= E (+ 1 with shared slots: column E is the gate of the experts every row uses);
+// ids and weights [T][top + shared].
+extern "C" int tie_moe_route(const float* logits, int row, const float* correction, int T, int E, int groups, int keep,
+                             int top, int sigmoid_scores, int group_top, int renormalize, float renorm_eps,
+                             float weight_scale, int shared, int* ids, float* weights, hipStream_t stream) {
   if (T <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || groups <= 0 || E % groups != 0 || keep <= 0 || keep > groups ||
-      top <= 0 || top > E)
+      top <= 0 || top > E || group_top <= 0 || group_top > MOE_MAX_GROUP_TOP || shared < 0 ||
+      row < E + (shared > 0 ? 1 : 0))
     return TIE_BAD_ARGUMENT;
-  const size_t shared = sizeof(float) * (2 * static_cast<size_t>(E) + groups);
-  moe_route_kernel<<<T, TIE_WAVE, shared, stream>>>(logits, correction, E, groups, keep, top, ids, weights);
+  const size_t lds = sizeof(float) * (2 * static_cast<size_t>(E) + groups);
+  moe_route_kernel<<<T, TIE_WAVE, lds, stream>>>(logits, row, correction, E, groups, keep, top, sigmoid_scores,
+                                                 group_top, renormalize, renorm_eps, weight_scale, shared, ids,
+                                                 weights);
   return tie_launch_status();
 }
 
@@ -191,14 +248,19 @@ extern "C" int tie_moe_align(const int* ids, int slots, int real, int tile_rows,
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
-// GATED: x rows are gathered (row = slot_at[place] / top), w_a and w_b are the gate and up weights
-// [real][N][K], out[place][c] = silu(a) * b. Otherwise x rows are the places themselves (act [slots][K]),
-// w_a is the down weight and out[place][c] = a.
-template <typename TX, typename TW, typename TO, bool GATED>
+// MODE 1 (gated): x rows are gathered (row = slot_at[place] / top), w_a and w_b are the gate and up weights
+// [real][N][K], out[place][c] = silu(a) * b. MODE 2 (experts without a gate): rows gathered likewise, w_a the up
+// weight, out[place][c] = relu(a)^2. MODE 0: x rows are the places themselves (act [slots][K]), w_a is the down
+// weight and out[place][c] = a.
+__device__ __forceinline__ float relu_squared_f(float a) { const float r = fmaxf(a, 0.f); return r * r; }
+
+template <typename TX, typename TW, typename TO, int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
     const TX* __restrict__ x, const TW* __restrict__ w_a, const TW* __restrict__ w_b, TO* __restrict__ out,
     const int* __restrict__ offsets, const int* __restrict__ slot_at, const int* __restrict__ tiles,
     const int* __restrict__ num_tiles, int top, int N, int K) {
+  constexpr bool GATED = MODE == 1;
+  constexpr bool GATHER = MODE != 0;
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;
   __shared__ float xs[GK][GR + 4];
@@ -210,7 +272,7 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
   const int rows = min(GR, offsets[e + 1] - place0);
   const int col0 = blockIdx.y * GC;
   const int tid = threadIdx.x;
-  if (tid < GR) src[tid] = tid < rows ? (GATED ? slot_at[place0 + tid] / top : place0 + tid) : -1;
+  if (tid < GR) src[tid] = tid < rows ? (GATHER ? slot_at[place0 + tid] / top : place0 + tid) : -1;
   __syncthreads();
   const TW* wa = w_a + static_cast<size_t>(e) * N * K;
   const TW* wb = GATED ? w_b + static_cast<size_t>(e) * N * K : nullptr;
@@ -263,7 +325,8 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
     for (int j = 0; j < 4; ++j) {
       const int c = col0 + tx * 4 + j;
       if (c >= N) continue;
-      const float v = GATED ? silu_f(acc_a[i][j]) * acc_b[i][j] : acc_a[i][j];
+      const float v = GATED ? silu_f(acc_a[i][j]) * acc_b[i][j]
+                            : (MODE == 2 ? relu_squared_f(acc_a[i][j]) : acc_a[i][j]);
       store_from_float(out + static_cast<size_t>(place0 + r) * N + c, v);
     }
   }
@@ -272,11 +335,13 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
 extern "C" int tie_moe_generic_tile_rows() { return GR; }
 
 // gated = 1: out [slots][N] of out_dtype = silu(x Wa^T) * (x Wb^T) over gathered rows of x [T][K];
+// gated = 2: out [slots][N] of out_dtype = relu(x Wa^T)^2 over gathered rows of x [T][K];
 // gated = 0: out [slots][N] = x Wa^T over x [slots][K]. Weights [real][N][K].
 extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a, const void* w_b, int w_dtype, void* out,
                                     int out_dtype, int gated, const int* offsets, const int* slot_at, const int* tiles,
                                     const int* num_tiles, int max_tiles, int top, int N, int K, hipStream_t stream) {
-  if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || (gated && w_b == nullptr)) return TIE_BAD_ARGUMENT;
+  if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || gated < 0 || gated > 2 || (gated == 1 && w_b == nullptr))
+    return TIE_BAD_ARGUMENT;
   if ((x_dtype | w_dtype | out_dtype) & ~1) return TIE_BAD_ARGUMENT;
   const dim3 grid(max_tiles, (N + GC - 1) / GC);
   if (grid.y > 65535) return TIE_BAD_ARGUMENT;
@@ -284,10 +349,11 @@ extern "C" int tie_moe_gemm_generic(const void* x, int x_dtype, const void* w_a,
   moe_gemm_generic_kernel<TX, TW, TO, G><<<grid, 256, 0, stream>>>(                                                \
       static_cast<const TX*>(x), static_cast<const TW*>(w_a), static_cast<const TW*>(w_b), static_cast<TO*>(out), \
       offsets, slot_at, tiles, num_tiles, top, N, K)
-#define LAUNCH(TX, TW, TO)             \
-  {                                    \
-    if (gated) LAUNCH_G(TX, TW, TO, true); \
-    else LAUNCH_G(TX, TW, TO, false);  \
+#define LAUNCH(TX, TW, TO)                    \
+  {                                           \
+    if (gated == 1) LAUNCH_G(TX, TW, TO, 1);  \
+    else if (gated == 2) LAUNCH_G(TX, TW, TO, 2); \
+    else LAUNCH_G(TX, TW, TO, 0);             \
   }
   const int key = x_dtype * 4 + w_dtype * 2 + out_dtype;
   switch (key) {
@@ -329,12 +395,14 @@ __device__ __forceinline__ moe_u32x4_t moe_load8(const bf16_t* p, bool in_range)
   return in_range ? *reinterpret_cast<const moe_u32x4_t*>(p) : moe_u32x4_t{0u, 0u, 0u, 0u};
 }
 
-template <int MT, int NT, bool GATED>
+template <int MT, int NT, int MODE>
 __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w_a, const bf16_t* __restrict__ w_b,
     void* __restrict__ out, const int* __restrict__ offsets, const int* __restrict__ slot_at,
     const int* __restrict__ tiles, const int* __restrict__ num_tiles, int top, int N, int K) {
   static_assert(MT == 1 || MT == 4 || MT == 8, "one x tile a wave, or MT / 4 loaded by each of the four waves");
+  constexpr bool GATED = MODE == 1;       // two weights, silu(a) * b
+  constexpr bool GATHER = MODE != 0;      // rows of x gathered by slot; the activations go out as bfloat16
   constexpr int OWN = MT == 1 ? 1 : MT / 4;                  // x fragments this wave loads a k-block
   const int tile = blockIdx.x;
   if (tile >= *num_tiles) return;                            // the whole workgroup leaves
@@ -357,7 +425,7 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
   for (int o = 0; o < OWN; ++o) {
     const int own_row = (MT == 1 ? 0 : wave * OWN + o) * 16 + r16;
     const int own_place = place0 + (own_row < rows ? own_row : 0);
-    const size_t src = GATED ? static_cast<size_t>(slot_at[own_place] / top) : static_cast<size_t>(own_place);
+    const size_t src = GATHER ? static_cast<size_t>(slot_at[own_place] / top) : static_cast<size_t>(own_place);
     xr[o] = x + src * K + quad * 8;
   }
   const bf16_t* wa[NT];
@@ -450,8 +518,10 @@ __global__ __launch_bounds__(256) void moe_gemm_bf16_kernel(
       const size_t at = static_cast<size_t>(place0 + r) * N + c;
       float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = GATED ? silu_f(acc_a[mt][nt][i]) * acc_b[mt][nt][i] : acc_a[mt][nt][i];
-      if (GATED) {
+      for (int i = 0; i < 4; ++i)
+        v[i] = GATED ? silu_f(acc_a[mt][nt][i]) * acc_b[mt][nt][i]
+                     : (MODE == 2 ? relu_squared_f(acc_a[mt][nt][i]) : acc_a[mt][nt][i]);
+      if (GATHER) {
         bf16_t* o = static_cast<bf16_t*>(out) + at;
         if (c + 3 < N && N % 4 == 0) {
           uint2 packed = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
@@ -479,16 +549,17 @@ extern "C" int tie_moe_bf16_tile_rows(int slots, int real) {
 }
 
 // bfloat16 x and weights; gated = 1: out bfloat16 [slots][N] = silu(x Wa^T) * (x Wb^T) over gathered rows of x;
+// gated = 2: out bfloat16 [slots][N] = relu(x Wa^T)^2 over gathered rows of x;
 // gated = 0: out float32 [slots][N] = x Wa^T over x [slots][K]. tile_rows (16, 64 or 128) as given to tie_moe_align.
 extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b, void* out, int gated,
                                  const int* offsets, const int* slot_at, const int* tiles, const int* num_tiles,
                                  int max_tiles, int tile_rows, int top, int N, int K, hipStream_t stream) {
-  if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || (gated && w_b == nullptr) ||
-      (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
+  if (max_tiles <= 0 || top <= 0 || N <= 0 || K <= 0 || K % 8 != 0 || gated < 0 || gated > 2 ||
+      (gated == 1 && w_b == nullptr) || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128) || reinterpret_cast<uintptr_t>(x) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(w_a) % 16 != 0 || reinterpret_cast<uintptr_t>(w_b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(out) % 16 != 0)
     return TIE_BAD_ARGUMENT;
-  const int columns = tile_rows == 16 ? 16 : (tile_rows == 128 && gated ? 128 : 256);   // of a workgroup
+  const int columns = tile_rows == 16 ? 16 : (tile_rows == 128 && gated == 1 ? 128 : 256);   // of a workgroup
   const dim3 grid(max_tiles, (N + columns - 1) / columns);
   if (grid.y > 65535) return TIE_BAD_ARGUMENT;
 #define LAUNCH_B(MT, NT, G)                                                                                  \
@@ -497,11 +568,11 @@ extern "C" int tie_moe_gemm_bf16(const void* x, const void* w_a, const void* w_b
                                                             static_cast<const bf16_t*>(w_b), out, offsets,   \
                                                             slot_at, tiles, num_tiles, top, N, K)
   if (tile_rows == 128) {
-    if (gated) LAUNCH_B(8, 2, true); else LAUNCH_B(8, 4, false);
+    if (gated == 1) LAUNCH_B(8, 2, 1); else if (gated == 2) LAUNCH_B(8, 4, 2); else LAUNCH_B(8, 4, 0);
   } else if (tile_rows == 64) {
-    if (gated) LAUNCH_B(4, 4, true); else LAUNCH_B(4, 4, false);
+    if (gated == 1) LAUNCH_B(4, 4, 1); else if (gated == 2) LAUNCH_B(4, 4, 2); else LAUNCH_B(4, 4, 0);
   } else {
-    if (gated) LAUNCH_B(1, 1, true); else LAUNCH_B(1, 1, false);
+    if (gated == 1) LAUNCH_B(1, 1, 1); else if (gated == 2) LAUNCH_B(1, 1, 2); else LAUNCH_B(1, 1, 0);
   }
 #undef LAUNCH_B
   return tie_launch_status();

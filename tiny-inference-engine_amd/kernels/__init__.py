@@ -61,6 +61,7 @@ _SOURCES = {
     "hyper": ("tie_hyper", "hyper.hip"),
     "delta_rule": ("tie_delta_rule", "delta_rule.hip"),
     "latent": ("tie_latent", "latent.hip"),
+    "pointwise": ("tie_pointwise", "pointwise.hip"),
 }
 # libraries compiled once per head size: key -> (file stem prefix, source)
 _PER_HEAD_DIM = {
@@ -108,7 +109,8 @@ _SIGNATURES = {
         "tie_argmax_static": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_void],
     },
     "moe": {
-        "tie_moe_route": [_c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void],
+        "tie_moe_route": [_c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                          _c_float, _c_float, _c_int, _c_void, _c_void, _c_void],
         "tie_moe_max_tiles": [_c_int, _c_int, _c_int],
         "tie_moe_align": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void, _c_void],
         "tie_moe_generic_tile_rows": [],
@@ -126,7 +128,7 @@ _SIGNATURES = {
     "attention_generic": {
         "tie_paged_attention_generic": [_c_void, _c_int, _c_void, _c_void, _c_int, _c_void, _c_int, _c_void, _c_void,
                                         _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
-                                        _c_float, _c_int, _c_int, _c_void, _c_void],
+                                        _c_float, _c_int, _c_int, _c_int, _c_void, _c_void],
     },
     "recurrent": {
         "tie_decay_attention_scan": [_c_void, _c_int, _c_void, _c_void, _c_void, _c_void, _c_void, _c_int, _c_int,
@@ -153,8 +155,14 @@ _SIGNATURES = {
         "tie_grouped_gated_rms_norm": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_void, _c_int, _c_int,
                                        _c_int, _c_int, _c_void],
     },
+    "pointwise": {
+        "tie_dynamic_tanh": [_c_void, _c_void, _c_long, _c_int, _c_void, _c_void, _c_void, _c_void, _c_int, _c_void,
+                             _c_int, _c_int, _c_int, _c_void],
+        "tie_token_gate": [_c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void],
+    },
     "latent": {
-        "tie_latent_prepare": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
+        "tie_rms_norm_columns": [_c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_int, _c_void],
+        "tie_latent_prepare": [_c_void, _c_int, _c_void, _c_int, _c_void, _c_float, _c_void, _c_int, _c_int, _c_void, _c_void, _c_void,
                                _c_int, _c_int, _c_int, _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                _c_int, _c_void],
         "tie_head_linear": [_c_void, _c_int, _c_int, _c_int, _c_void, _c_int, _c_void, _c_int, _c_int, _c_int, _c_void,
@@ -1005,13 +1013,15 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
                             query_start: torch.Tensor, context_lens: torch.Tensor, block_tables: torch.Tensor,
                             seq_of_row: torch.Tensor, num_heads: int, scale: float,
                             window: Optional[int] = None, softcap: Optional[float] = None,
-                            chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> None:
+                            chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None,
+                            keep_first: int = 0) -> None:
     """Causal attention of every query row over its sequence's cached keys (float32 arithmetic, any sizes).
 
     ``softcap`` c (None or 0: none): scores become ``c * tanh(scale * q.k / c)`` before the softmax.
     ``chunk`` n: a query at position p reads the keys from ``p - p % n`` on (causal chunks counted from the
     sequence's position 0) instead of a sliding ``window``. ``sinks`` (float32 ``[heads]``): ``exp(sinks[h])``
-    is one more term of head h's softmax denominator."""
+    is one more term of head h's softmax denominator. ``keep_first`` f (beside a window): the keys of positions
+    below f are read as well, at their true positions."""
     _gpu(q, "queries")
     _gpu(out, "attention output")
     _gpu(k_cache, "k cache")
@@ -1037,13 +1047,15 @@ def paged_attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
         raise InvalidArgument(f"block tables {list(block_tables.shape)} do not cover {S} sequences")
     if window and chunk:
         raise InvalidArgument("attention takes a sliding window or causal chunks, not both")
+    if keep_first and not window:
+        raise InvalidArgument("first positions are kept beside a sliding window only")
     if sinks is not None:
         _f32(sinks, "attention sinks", (H,))
     _call(_lib("attention_generic").tie_paged_attention_generic, "paged_attention_generic",
         q.data_ptr(), _code(q, "queries"), k_cache.data_ptr(), v_cache.data_ptr(), _cache_code(k_cache, q, "k cache"),
         out.data_ptr(), _code(out, "attention output"), query_start.data_ptr(), context_lens.data_ptr(),
         block_tables.data_ptr(), seq_of_row.data_ptr(), T, H, KVH, Dh, bs, block_tables.shape[1], float(scale),
-        float(softcap or 0.0), int(window or 0), int(chunk or 0), _ptr(sinks), _stream())
+        float(softcap or 0.0), int(window or 0), int(chunk or 0), int(keep_first or 0), _ptr(sinks), _stream())
 
 
 _argmax_workspace = {}
@@ -1523,7 +1535,7 @@ def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_conte
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step, batch,
                     num_heads: int, scale: float, window: Optional[int] = None, scratch=None,
                     softcap: Optional[float] = None, chunk: Optional[int] = None,
-                    sinks: Optional[torch.Tensor] = None) -> None:
+                    sinks: Optional[torch.Tensor] = None, keep_first: int = 0) -> None:
     """Causal attention over the paged cache for one step's batch, on the fastest kernel that takes it.
 
     ``step`` is the cache group's view of the step (block tables), ``batch`` the step's arrays
@@ -1533,7 +1545,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     NB, KVH, bs, Dh = k_cache.shape
     fast = (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and Dh in MFMA_HEAD_DIMS
             and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
-    reach = window or chunk      # the most keys a query reads: what the shares of a sequence's keys are planned by
+    if keep_first and not window:
+        raise InvalidArgument("first positions are kept beside a sliding window only")
+    if keep_first:
+        fast = False           # kept first positions: the generic kernel walks them
+    reach = (window + keep_first if window else None) or chunk      # the most keys a query reads: what the shares of a sequence's keys are planned by
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
         nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
@@ -1595,7 +1611,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
             paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                                    batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks)
+                                    batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks, keep_first)
             return
         if items is not None:
             rows = q.shape[0]
@@ -1611,7 +1627,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                                    merge_rows if nsplit > 1 else None, softcap=softcap, chunk=chunk, sinks=sinks)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
-                            batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks)
+                            batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks, keep_first)
 
 
 # ------------------------------------------------------------------ mixers with a state of fixed size
@@ -1746,27 +1762,41 @@ def min_gru_scan(proj: torch.Tensor, out: torch.Tensor, state: torch.Tensor, que
 MOE_MAX_EXPERTS = 1024       # MOE_MAX_EXPERTS of csrc/moe.hip
 
 
-def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
-              ids: torch.Tensor, weights: torch.Tensor) -> None:
-    """The router's choice for every row of float32 ``logits [T, E]``.
+MOE_MAX_GROUP_TOP = 8         # MOE_MAX_GROUP_TOP of csrc/moe.hip
 
-    ``s = softmax(logits)``; the choice looks at ``s + correction``: the experts form ``groups`` equal groups of
-    neighbours, a group scores its best member, only members of the ``keep`` best groups stay eligible, and the
-    ``top`` best of those are chosen (ties to the lower index) into ``ids`` int32 ``[T, top]``; ``weights``
-    float32 ``[T, top]`` are ``s`` at the chosen, not renormalised.
+
+def moe_route(logits: torch.Tensor, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
+              ids: torch.Tensor, weights: torch.Tensor, scoring: str = "softmax", group_top: int = 1,
+              renormalize: bool = False, renorm_eps: float = 0.0, weight_scale: float = 1.0, shared: int = 0) -> None:
+    """The router's choice for every row of float32 ``logits [T, E]`` (``[T, E + 1]`` with ``shared``).
+
+    ``s = softmax(logits)`` over the experts, or with ``scoring`` ``"sigmoid"`` ``sigmoid(logits)`` expert by expert;
+    the choice looks at ``s + correction``: the experts form ``groups`` equal groups of neighbours, a group scores
+    the sum of its ``group_top`` best members (1: its best member), only members of the ``keep`` best groups stay
+    eligible, and the ``top`` best of those are chosen (ties to the lower index) into ``ids`` int32; ``weights``
+    float32 are ``s`` at the chosen, with ``renormalize`` divided by their sum + ``renorm_eps``, times
+    ``weight_scale``. ``shared`` n: both arrays are ``[T, top + n]``, the last n slots of a row name the experts
+    ``E .. E + n - 1`` (experts every row uses) with the weight ``sigmoid(logits[:, E])``.
     """
     _f32(logits, "router logits")
-    T, E = logits.shape
+    T, row = logits.shape
+    E = row - (1 if shared else 0)
+    slots = top + shared
     if correction is not None:
         _f32(correction, "the choice's correction", (E,))
     _i32(ids, "chosen experts")
-    _f32(weights, "routing weights", (T, top))
-    if tuple(ids.shape) != (T, top):
-        raise InvalidArgument(f"chosen experts {list(ids.shape)} do not fit {[T, top]}")
-    if not 0 < E <= MOE_MAX_EXPERTS or groups <= 0 or E % groups or not 0 < keep <= groups or not 0 < top <= E:
-        raise InvalidArgument(f"moe_route: {E} experts (at most {MOE_MAX_EXPERTS}) in {groups} groups, {keep} kept, top {top}")
-    _call(_lib("moe").tie_moe_route, "moe_route", logits.data_ptr(), _ptr(correction), T, E, groups, keep, top,
-          ids.data_ptr(), weights.data_ptr(), _stream())
+    _f32(weights, "routing weights", (T, slots))
+    if tuple(ids.shape) != (T, slots):
+        raise InvalidArgument(f"chosen experts {list(ids.shape)} do not fit {[T, slots]}")
+    if scoring not in ("softmax", "sigmoid"):
+        raise InvalidArgument(f"router scoring '{scoring}' (supported: softmax, sigmoid)")
+    if not 0 < E <= MOE_MAX_EXPERTS or groups <= 0 or E % groups or not 0 < keep <= groups or not 0 < top <= E or \
+            not 0 < group_top <= MOE_MAX_GROUP_TOP or shared < 0:
+        raise InvalidArgument(f"moe_route: {E} experts (at most {MOE_MAX_EXPERTS}) in {groups} groups scored by their "
+                              f"{group_top} best, {keep} kept, top {top}")
+    _call(_lib("moe").tie_moe_route, "moe_route", logits.data_ptr(), row, _ptr(correction), T, E, groups, keep, top,
+          int(scoring == "sigmoid"), int(group_top), int(bool(renormalize)), float(renorm_eps), float(weight_scale),
+          int(shared), ids.data_ptr(), weights.data_ptr(), _stream())
 
 
 class ExpertRows:
@@ -1829,22 +1859,30 @@ def _moe_weights(w: torch.Tensor, real: int, name: str):
     return w.shape[1], w.shape[2]
 
 
-def moe_gate_up(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, rows: ExpertRows, act: torch.Tensor) -> None:
-    """``act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T)`` for every sorted slot: ``x [T, K]``, weights ``[real, F, K]``."""
+def moe_gate_up(x: torch.Tensor, w_gate: Optional[torch.Tensor], w_up: torch.Tensor, rows: ExpertRows,
+                act: torch.Tensor) -> None:
+    """``act[place] = silu(x[row] Wg_e^T) * (x[row] Wu_e^T)`` for every sorted slot: ``x [T, K]``, weights
+    ``[real, F, K]``. Without gate weights (``w_gate`` None) the experts have no gate and the activation is the square
+    of relu: ``act[place] = relu(x[row] Wu_e^T)^2``."""
     _gpu(x, "the experts' input rows")
     _gpu(act, "the experts' activations")
-    F_, K = _moe_weights(w_gate, rows.real, "gate weights")
-    if tuple(w_up.shape) != tuple(w_gate.shape) or w_up.dtype != w_gate.dtype or not w_up.is_contiguous():
+    F_, K = _moe_weights(w_up, rows.real, "up weights")
+    mode = 2 if w_gate is None else 1
+    if w_gate is not None and (tuple(w_up.shape) != tuple(w_gate.shape) or w_up.dtype != w_gate.dtype or
+                               not w_gate.is_contiguous() or not w_gate.is_cuda):
         raise InvalidArgument("gate and up weights must be alike")
+    first = w_up if w_gate is None else w_gate
     if x.dim() != 2 or x.shape[1] != K or x.shape[0] * rows.top != rows.slots or tuple(act.shape) != (rows.slots, F_):
-        raise InvalidArgument(f"moe_gate_up: rows {list(x.shape)}, activations {list(act.shape)}, weights {list(w_gate.shape)}")
-    if _moe_on_matrix_cores(rows, x, w_gate, act, True):
-        _call(_lib("moe").tie_moe_gemm_bf16, "moe_gate_up", x.data_ptr(), w_gate.data_ptr(), w_up.data_ptr(),
-              act.data_ptr(), 1, rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(),
+        raise InvalidArgument(f"moe_gate_up: rows {list(x.shape)}, activations {list(act.shape)}, weights {list(w_up.shape)}")
+    if _moe_on_matrix_cores(rows, x, first, act, True):
+        _call(_lib("moe").tie_moe_gemm_bf16, "moe_gate_up", x.data_ptr(), first.data_ptr(),
+              w_up.data_ptr() if w_gate is not None else None,
+              act.data_ptr(), mode, rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(),
               rows.num_tiles.data_ptr(), rows.max_tiles, rows.tile_rows, rows.top, F_, K, _stream())
         return
-    _call(_lib("moe").tie_moe_gemm_generic, "moe_gate_up", x.data_ptr(), _code(x, "rows"), w_gate.data_ptr(),
-          w_up.data_ptr(), _code(w_gate, "gate weights"), act.data_ptr(), _code(act, "activations"), 1,
+    _call(_lib("moe").tie_moe_gemm_generic, "moe_gate_up", x.data_ptr(), _code(x, "rows"), first.data_ptr(),
+          w_up.data_ptr() if w_gate is not None else None, _code(first, "expert weights"), act.data_ptr(),
+          _code(act, "activations"), mode,
           rows.offsets.data_ptr(), rows.slot_at.data_ptr(), rows.tiles.data_ptr(), rows.num_tiles.data_ptr(),
           rows.max_tiles, rows.top, F_, K, _stream())
 
@@ -1881,6 +1919,59 @@ def moe_combine(routed: RoutedParts, out: torch.Tensor, accumulate: bool = False
     _call(_lib("moe").tie_moe_combine, "moe_combine", routed.parts.data_ptr(), routed.where.data_ptr(),
           routed.weights.data_ptr(), routed.self_rows.data_ptr(), _code(routed.self_rows, "input rows"),
           out.data_ptr(), T, top, n, int(accumulate), _stream())
+
+
+# ------------------------------------------------- kernels without statistics over a row
+def dynamic_tanh(x: torch.Tensor, alpha: Optional[torch.Tensor], weight: Optional[torch.Tensor],
+                 bias: Optional[torch.Tensor], out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                 owed: Optional[torch.Tensor] = None) -> None:
+    """``out = tanh(alpha * x) * weight + bias`` over rows of the float32 stream ``x`` (``alpha`` a float32 tensor of
+    one element, read on the device). ``rows``: gather these rows. ``owed`` (float32 ``[planes, T, n]``): partial sums
+    still owed to the stream, added into ``x`` in plane order in the same pass. Without ``alpha`` the function is
+    left out: ``out = x`` in the output's type (with the owed sums added)."""
+    _f32(x, "the stream")
+    _gpu(out, "dynamic_tanh output")
+    n = x.shape[-1]
+    R = out.numel() // n if n else 0
+    if out.shape[-1] != n or (rows is None and x.numel() != out.numel()):
+        raise InvalidArgument(f"dynamic_tanh output {list(out.shape)} does not match input {list(x.shape)}")
+    plain = alpha is None
+    if not plain:
+        _f32(alpha, "dynamic_tanh alpha", (1,))
+        _f32(weight, "dynamic_tanh weight", (n,))
+        _f32(bias, "dynamic_tanh bias", (n,))
+    planes = 0
+    if owed is not None:
+        _f32(owed, "owed partial sums")
+        if rows is not None or owed.dim() != 3 or tuple(owed.shape[1:]) != tuple(x.shape):
+            raise InvalidArgument(f"owed sums {list(owed.shape)} do not fit the stream {list(x.shape)}")
+        planes = owed.shape[0]
+    if rows is not None:
+        _i32(rows, "dynamic_tanh rows", R)
+    if R == 0:
+        return
+    if R > MAX_STEP_TOKENS:
+        raise InvalidArgument(f"a step of {R} rows exceeds the {MAX_STEP_TOKENS} this kernel takes")
+    _call(_lib("pointwise").tie_dynamic_tanh, "dynamic_tanh", x.data_ptr(), _ptr(owed), x.numel(), planes,
+          _ptr(alpha), _ptr(weight), _ptr(bias), out.data_ptr(), _code(out, "dynamic_tanh output"), _ptr(rows), R, n,
+          int(plain), _stream())
+
+
+def token_gate(gate: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, first: int, out: torch.Tensor) -> None:
+    """``out[t, j] = gelu_tanh(gate[t, j]) * table[tokens[t], first + j]``: ``gate`` float32 ``[T, dim]``, ``table``
+    ``[vocab, columns]`` (every layer a range of columns of its own), ``out`` ``[T, dim]``."""
+    _f32(gate, "the gate's sums")
+    _gpu(table, "the per-token table")
+    _gpu(out, "gated token rows")
+    T, dim = gate.shape
+    _i32(tokens, "token ids", T)
+    if table.dim() != 2 or first < 0 or first + dim > table.shape[1] or tuple(out.shape) != (T, dim):
+        raise InvalidArgument(f"token_gate: table {list(table.shape)}, columns {first} .. {first + dim}, out {list(out.shape)}")
+    if T == 0:
+        return
+    _call(_lib("pointwise").tie_token_gate, "token_gate", gate.data_ptr(), tokens.data_ptr(), table.data_ptr(),
+          _code(table, "the per-token table"), table.shape[1], int(first), out.data_ptr(),
+          _code(out, "gated token rows"), T, dim, _stream())
 
 
 # ------------------------------------------------- layer norm, hyper-connections
@@ -2117,20 +2208,30 @@ def grouped_gated_rms_norm(o: torch.Tensor, weight: torch.Tensor, eps: float, ga
 def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor, eps: float, angles: Optional[torch.Tensor],
                    rotary_dim: int, pairing: str, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                    v_cache: Optional[torch.Tensor], block_size: int, write_kv: bool, q_plain: torch.Tensor,
-                   q_latent: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: int) -> None:
+                   q_latent: torch.Tensor, heads: int, dim: int, rot_dim: int, kv_rank: int,
+                   latent_rows: Optional[torch.Tensor] = None) -> None:
     """Cache rows and query parts of a latent attention from the projection's float32 rows
     ``[q: H x (dim + rot_dim) | latent (kv_rank) | rotated key part (rot_dim) | ...]``.
 
     The latent is RMS-normed with ``latent_weight``; the key cache (one head of size D >= kv_rank + rot_dim) gets
     ``[latent | rotated key part | zeros]``, the value cache ``[latent | zeros]``. ``q_plain`` ``[T, H dim]`` gets
     the unrotated query parts, ``q_latent`` ``[T, H D]`` the rotated ones at columns ``kv_rank ..`` of every head
-    (zeros behind; columns below ``kv_rank`` are left for the product that takes the plain parts there)."""
+    (zeros behind; columns below ``kv_rank`` are left for the product that takes the plain parts there).
+    ``latent_rows`` (float32 ``[T, >= kv_rank + rot_dim]``, rows possibly further apart): the latent and the key part
+    where they do not follow the queries in ``proj`` (queries that come from a product of their own)."""
     _gpu_strided(proj, "projected rows")
     T = proj.shape[0]
     H, d, r, kr = heads, dim, rot_dim, kv_rank
     D = q_latent.shape[1] // H
-    if proj.dtype != torch.float32 or proj.shape[1] < H * (d + r) + kr + r or proj.stride(1) != 1:
+    if proj.dtype != torch.float32 or proj.shape[1] < H * (d + r) + (0 if latent_rows is not None else kr + r) or \
+            proj.stride(1) != 1:
         raise InvalidArgument(f"projected rows {list(proj.shape)} {proj.dtype} do not hold the queries and the latent")
+    if latent_rows is not None:
+        _gpu_strided(latent_rows, "latent rows")
+        if latent_rows.dtype != torch.float32 or latent_rows.dim() != 2 or latent_rows.shape[0] != T or \
+                latent_rows.shape[1] < kr + r or latent_rows.stride(1) != 1:
+            raise InvalidArgument(f"latent rows {list(latent_rows.shape)} {latent_rows.dtype} do not hold the latent "
+                                  f"and the key part of {T} tokens")
     _gpu(q_plain, "plain query parts")
     _gpu(q_latent, "latent queries")
     if tuple(q_plain.shape) != (T, H * d) or tuple(q_latent.shape) != (T, H * D) or D < kr + r or \
@@ -2148,11 +2249,28 @@ def latent_prepare(proj: torch.Tensor, latent_weight: torch.Tensor, eps: float, 
         cache_code = _cache_code(k_cache, q_plain, "k cache")
     if T == 0:
         return
-    _call(_lib("latent").tie_latent_prepare, "latent_prepare", proj.data_ptr(), proj.stride(0), latent_weight.data_ptr(),
+    _call(_lib("latent").tie_latent_prepare, "latent_prepare", proj.data_ptr(), proj.stride(0),
+          latent_rows.data_ptr() if latent_rows is not None else None,
+          latent_rows.stride(0) if latent_rows is not None else 0, latent_weight.data_ptr(),
           float(eps), _ptr(angles) if rotary_dim else None, int(rotary_dim), int(pairing == "interleaved"),
           _ptr(slots) if write_kv else None, _ptr(k_cache) if write_kv else None, _ptr(v_cache) if write_kv else None,
           cache_code, block_size, int(write_kv), q_plain.data_ptr(), q_latent.data_ptr(), _code(q_plain, "queries"),
           T, H, d, r, kr, D, _stream())
+
+
+def rms_norm_columns(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """``out = RMSNorm(x) * weight`` over float32 rows ``x [T, n]`` that may lie further apart than ``n`` (the first
+    columns of wider rows); ``out`` ``[T, n]`` dense."""
+    _gpu_strided(x, "rows to norm")
+    _gpu(out, "normed rows")
+    if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1 or tuple(out.shape) != tuple(x.shape):
+        raise InvalidArgument(f"rms_norm_columns: rows {list(x.shape)} {x.dtype}, out {list(out.shape)}")
+    T, n = x.shape
+    _f32(weight, "norm weight", (n,))
+    if T == 0:
+        return
+    _call(_lib("latent").tie_rms_norm_columns, "rms_norm_columns", x.data_ptr(), x.stride(0), weight.data_ptr(),
+          float(eps), out.data_ptr(), _code(out, "normed rows"), T, n, _stream())
 
 
 def head_linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:

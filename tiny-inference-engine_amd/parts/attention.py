@@ -33,6 +33,8 @@ Further parameters, for architectures that have them (absent or None: not applie
 * ``chunk`` n: instead of a sliding window, a query at position p sees the keys ``j <= p`` of its own chunk,
   ``floor(j / n) = floor(p / n)``, chunks counted from the sequence's position 0 (not from where a prompt was cut).
   The cache gives back the pages of chunks a request has left behind.
+* ``keep_first`` f (beside a ``window``): a query also sees the keys of positions below f, at their true positions
+  (for the rotation and for distances), however far back they lie; the cache keeps their pages to the request's end.
 * ``sink`` (a tensor name, one float per query head): ``exp(sink[h])`` is one more term of head h's softmax
   denominator; it has no key and no value and is not scaled.
 * ``values_are_keys``: there is no value projection; the values are the keys as projected (with their bias), before
@@ -82,6 +84,9 @@ class PagedAttention(Mixer):
         self.chunk: Optional[int] = int(params["chunk"]) if params.get("chunk") else None
         if self.window and self.chunk:
             raise InvalidArgument("attention takes a sliding window or causal chunks, not both")
+        self.keep_first = int(params.get("keep_first") or 0)
+        if self.keep_first < 0 or (self.keep_first and not self.window):
+            raise InvalidArgument("first positions are kept beside a sliding window only")
         self.sink_name: Optional[str] = params.get("sink")
         self.sinks: torch.Tensor = None
         self.values_are_keys = bool(params.get("values_are_keys", False))
@@ -156,7 +161,7 @@ class PagedAttention(Mixer):
         return [self.position]
 
     def cache_need(self):
-        pages = PagedKV(self.num_kv_heads, self.head_dim, self.window, self.chunk)
+        pages = PagedKV(self.num_kv_heads, self.head_dim, self.window, self.chunk, self.keep_first)
         if self.taps > 1:
             return (pages, FixedState((self.taps - 1, self.q_dim + 2 * self.kv_dim)))
         return pages
@@ -312,7 +317,7 @@ class PagedAttention(Mixer):
             inv_freq, rotary_dim, pairing = table
             if (inv_freq is not None and not rows_first and rotary_dim == Dh and pairing == "rotate_half" and self.softcap is None
                     and self.value_mix is None and not self.values_are_keys and not self.chunk and self.sinks is None
-                    and self.qkv_bias is None
+                    and self.qkv_bias is None and not self.keep_first
                     and kernels.decode_attention_prepares(ctx.batch, q.dtype, cache.k_cache, H)):
                 # A step of single decoded tokens: the attention kernel sums the planes, norms and rotates its own
                 # queries and writes the newest keys and values itself: one kernel less.
@@ -349,5 +354,6 @@ class PagedAttention(Mixer):
 
         attn = ctx.scratch("attention.out", (T, self.q_dim))
         kernels.paged_attention(q, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale, self.window,
-                                scratch=ctx.scratch, softcap=self.softcap, chunk=self.chunk, sinks=self.sinks)
+                                scratch=ctx.scratch, softcap=self.softcap, chunk=self.chunk, sinks=self.sinks,
+                                keep_first=self.keep_first)
         return self._finish(ctx, attn, residual)

@@ -11,6 +11,12 @@ half alone (and needs that half's norm only).
 adding it (``forward(..., residual=None)``); the norm over the result, the addition to the stream and the norm
 that the stream meets next run as one kernel where the norms can (``Norm.add_normed``).
 
+``pre_norm_token_side`` is ``pre_norm`` followed by a third step that feeds every layer a vector of its own per
+token: with ``e = table[token]`` restricted to the layer's ``dim`` columns (``first .. first + dim`` of a table all
+layers share), ``g = gelu_tanh(W_gate x) * e`` from the stream itself (no norm before it), ``y = W_proj g`` and
+``x += y / sqrt(mean(y^2) + eps) * w``. Parameters: ``hidden``, ``dim``, ``vocab``, ``table`` (tensor name),
+``table_columns``, ``first``, ``eps``, ``names`` (``gate``, ``proj``, ``norm``).
+
 ``hyper_connections`` keeps ``streams`` copies of the residual instead of one. All start as the embedding's rows.
 Sub-layer q of a layer (its mixer, then its feed-forward) has three small tensors ``in`` ``[streams]``, ``out``
 ``[streams]`` and ``mix`` ``[streams, streams]`` (from, to): it reads ``u = sum_s in[s] x_s``, computes
@@ -30,6 +36,7 @@ import torch
 from .. import kernels
 from ..errors import InvalidArgument
 from .base import Block, StepContext, TensorSpec, register_part
+from .linear import Linear
 
 
 @register_part("block", "pre_norm")
@@ -54,6 +61,69 @@ class PreNormBlock(Block):
         missing = [n for n in needed if n not in layer.norms]
         if missing:
             raise InvalidArgument(f"a pre_norm block needs the norms {', '.join(needed)}; missing {', '.join(missing)}")
+
+
+@register_part("block", "pre_norm_token_side")
+class TokenSideBlock(PreNormBlock):
+    capturable = True
+    replayable = True
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.hidden = int(params["hidden"])
+        self.dim = int(params["dim"])
+        self.vocab = int(params["vocab"])
+        self.table_name = params["table"]
+        self.table_columns = int(params["table_columns"])
+        self.first = int(params["first"])
+        self.eps = float(params["eps"])
+        if self.dim <= 0 or self.first < 0 or self.first + self.dim > self.table_columns:
+            raise InvalidArgument(f"columns {self.first} .. {self.first + self.dim} do not lie in a per-token table of "
+                                  f"{self.table_columns} columns")
+        names = params["names"]
+        self.gate = Linear([names["gate"]], [self.dim], self.hidden)
+        self.proj = Linear([names["proj"]], [self.hidden], self.dim)
+        self.norm_name = names["norm"]
+        self.norm_weight: torch.Tensor = None
+        self.table: torch.Tensor = None          # this layer's columns of the shared table, [vocab, dim]
+
+    def tensors(self) -> List[TensorSpec]:
+        return self.gate.tensors() + self.proj.tensors() + [
+            TensorSpec(self.norm_name, (self.hidden,), "vector", ("one_plus_uniform", 0.1)),
+            TensorSpec(self.table_name, (self.vocab, self.table_columns), "matrix", ("normal", 0.5))]
+
+    def load(self, fetch, mode, device) -> None:
+        self.gate.load(fetch)
+        self.proj.load(fetch)
+        self.norm_weight = fetch(self.norm_name, "vector")
+        # a copy of the layer's own columns: a token's vector is then one piece of consecutive memory, and layers of
+        # one shape differ in addresses only
+        self.table = fetch(self.table_name, "matrix")[:, self.first:self.first + self.dim].contiguous()
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, layer, cache) -> None:
+        super().forward(ctx, x, layer, cache)
+        T = x.shape[0]
+        if ctx.act_dtype == torch.float32:
+            ctx.settle()
+            rows = x
+        else:
+            # the stream in the products' type, in the pass that adds what the feed-forward still owes it
+            if ctx._late is not None:
+                ctx.settle()
+            owed = ctx.take_owed(x)
+            rows = ctx.scratch("token_side.rows", (T, self.hidden), ctx.act_dtype)
+            ctx.set_row_scale(rows, None)
+            kernels.dynamic_tanh(x, None, None, None, rows, None, owed)
+        gate = ctx.scratch("token_side.gate", (T, self.dim), torch.float32)
+        self.gate(rows, gate, ctx=ctx)
+        gated = ctx.scratch("token_side.gated", (T, self.dim), ctx.act_dtype)
+        ctx.set_row_scale(gated, None)
+        kernels.token_gate(gate, ctx.batch.tokens, self.table, 0, gated)
+        y = self.proj.partial_planes(ctx, gated, "token_side.result_planes")
+        if y is None:
+            y = ctx.scratch("token_side.result", (T, self.hidden), torch.float32)
+            self.proj(gated, y, ctx=ctx)
+        kernels.norm_add_norm(y, self.norm_weight, self.eps, x)
 
 
 @register_part("block", "sandwich_norm")

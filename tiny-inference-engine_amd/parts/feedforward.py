@@ -28,6 +28,15 @@ result is the weighted sum of the chosen experts' results. Parameters: ``hidden`
 ``experts``, ``identity_experts``, ``top``, ``groups``, ``keep_groups``, ``scoring``, ``renormalize``, ``names``
 (``router``, ``correction`` or None, and lists ``gate``, ``up``, ``down`` with one name an expert).
 
+For designs that have them: ``scoring`` ``sigmoid`` (scores are ``sigmoid(logits)`` expert by expert);
+``group_top`` n (a group scores the sum of its n best members instead of its best); ``renormalize`` True (the
+weights are the chosen scores divided by their sum + ``renorm_eps``); ``weight_scale`` (a factor on the weights);
+``expert_activation`` ``relu_squared`` with no ``gate`` names (experts without a gate, ``down_e(relu(up_e h)^2)``);
+``shared`` ``{"intermediate", "up", "down", "gate_logit"}`` (and ``"gate"`` for gated experts): one more expert of the
+same form that every row uses, its result multiplied by ``sigmoid(w_gate_logit . h)``, one number a row. It runs as
+pieces of the routed experts' size among them (further experts that every row chooses, all with that weight), so
+the same launches carry it; its gate's logit is one more column of the router's product.
+
 Nothing of a step is read on the host: the rows are sorted by expert on the device and the experts' products
 run over a tile list that lives there (``kernels.moe_align``), so routed layers are recorded and replayed like
 dense ones.
@@ -171,64 +180,104 @@ class RoutedExperts(FeedForward):
         self.top = int(params["top"])
         self.groups = int(params.get("groups") or 1)
         self.keep_groups = int(params.get("keep_groups") or self.groups)
-        if params.get("scoring", "softmax") != "softmax":
-            raise UnsupportedError(f"router scoring '{params['scoring']}' (supported: softmax)")
-        if params.get("renormalize"):
-            raise UnsupportedError("renormalised routing weights are not implemented")
+        self.scoring = params.get("scoring") or "softmax"
+        if self.scoring not in ("softmax", "sigmoid"):
+            raise UnsupportedError(f"router scoring '{self.scoring}' (supported: softmax, sigmoid)")
+        self.group_top = int(params.get("group_top") or 1)
+        self.renormalize = bool(params.get("renormalize"))
+        self.renorm_eps = float(params.get("renorm_eps") or 0.0)
+        self.weight_scale = float(params.get("weight_scale") if params.get("weight_scale") is not None else 1.0)
+        names = params["names"]
+        self.gated = bool(names.get("gate"))
+        self.activation = params.get("expert_activation") or ("silu" if self.gated else "relu_squared")
+        if (self.gated and self.activation != "silu") or (not self.gated and self.activation != "relu_squared"):
+            raise UnsupportedError(f"experts {'with' if self.gated else 'without'} a gate and the activation "
+                                   f"'{self.activation}' (supported: silu with a gate, relu_squared without)")
         if self.experts <= 0 or self.identity < 0 or self.outputs > kernels.MOE_MAX_EXPERTS:
             raise InvalidArgument(f"a routed feed-forward takes 1 to {kernels.MOE_MAX_EXPERTS} experts, got "
                                   f"{self.experts} + {self.identity}")
         if self.outputs % self.groups or not 0 < self.keep_groups <= self.groups or \
-                not 0 < self.top <= self.keep_groups * (self.outputs // self.groups):
-            raise InvalidArgument(f"{self.outputs} experts in {self.groups} groups, {self.keep_groups} kept, top "
-                                  f"{self.top}: no such choice")
-        names = params["names"]
-        for key in ("gate", "up", "down"):
+                not 0 < self.top <= self.keep_groups * (self.outputs // self.groups) or \
+                not 0 < self.group_top <= kernels.MOE_MAX_GROUP_TOP:
+            raise InvalidArgument(f"{self.outputs} experts in {self.groups} groups scored by their {self.group_top} "
+                                  f"best, {self.keep_groups} kept, top {self.top}: no such choice")
+        for key in ("gate", "up", "down") if self.gated else ("up", "down"):
             if len(names[key]) != self.experts:
                 raise InvalidArgument(f"a routed feed-forward needs one '{key}' tensor name per expert")
         self.names = names
-        self.router = Linear([names["router"]], [self.outputs], self.hidden)
+        # The expert every row uses, cut into pieces of the routed experts' size that sit behind them.
+        self.shared = dict(params["shared"]) if params.get("shared") else None
+        self.shared_intermediate = int(self.shared["intermediate"]) if self.shared else 0
+        self.shared_pieces = -(-self.shared_intermediate // self.intermediate) if self.shared else 0
+        if self.shared:
+            if self.identity:
+                raise InvalidArgument("a shared expert beside experts that return their input is not supported")
+            if self.shared_intermediate <= 0 or self.experts + self.shared_pieces > kernels.MOE_MAX_EXPERTS:
+                raise InvalidArgument(f"a shared expert of inner size {self.shared_intermediate} does not fit")
+            router_names, router_sizes = [names["router"], self.shared["gate_logit"]], [self.outputs, 1]
+        else:
+            router_names, router_sizes = [names["router"]], [self.outputs]
+        self.router = Linear(router_names, router_sizes, self.hidden)
         self.correction: torch.Tensor = None
-        self.gate: torch.Tensor = None        # [experts, intermediate, hidden]
+        self.gate: torch.Tensor = None        # [experts (+ shared pieces), intermediate, hidden]
         self.up: torch.Tensor = None
-        self.down: torch.Tensor = None        # [experts, hidden, intermediate]
+        self.down: torch.Tensor = None        # [experts (+ shared pieces), hidden, intermediate]
 
     def tensors(self) -> List[TensorSpec]:
         specs = self.router.tensors()
         if self.names.get("correction"):
             specs.append(TensorSpec(self.names["correction"], (self.outputs,), "vector", ("normal", 0.02)))
+        inner = ("gate", "up") if self.gated else ("up",)
         for e in range(self.experts):
-            specs.append(TensorSpec(self.names["gate"][e], (self.intermediate, self.hidden), "matrix", ("normal", 0.02)))
-            specs.append(TensorSpec(self.names["up"][e], (self.intermediate, self.hidden), "matrix", ("normal", 0.02)))
+            for key in inner:
+                specs.append(TensorSpec(self.names[key][e], (self.intermediate, self.hidden), "matrix", ("normal", 0.02)))
             specs.append(TensorSpec(self.names["down"][e], (self.hidden, self.intermediate), "matrix", ("normal", 0.02)))
+        if self.shared:
+            for key in inner:
+                specs.append(TensorSpec(self.shared[key], (self.shared_intermediate, self.hidden), "matrix", ("normal", 0.02)))
+            specs.append(TensorSpec(self.shared["down"], (self.hidden, self.shared_intermediate), "matrix", ("normal", 0.02)))
         return specs
 
     def load(self, fetch, mode, device) -> None:
         self.router.load(fetch)
         if self.names.get("correction"):
             self.correction = fetch(self.names["correction"], "vector")
+        F_, pieces = self.intermediate, self.shared_pieces
 
-        def stack(key):
+        def stack(key, inner_rows: bool):
             parts = [fetch(n, "matrix") for n in self.names[key]]
+            if self.shared:
+                w = fetch(self.shared[key], "matrix")
+                # zero rows of an up (or gate) matrix give zero activations; they meet zero columns of the down matrix
+                wide = w.new_zeros((pieces * F_, self.hidden) if inner_rows else (self.hidden, pieces * F_))
+                if inner_rows:
+                    wide[:self.shared_intermediate] = w
+                    parts += list(wide.view(pieces, F_, self.hidden).unbind(0))
+                else:
+                    wide[:, :self.shared_intermediate] = w
+                    parts += list(wide.view(self.hidden, pieces, F_).unbind(1))
             if len({p.dtype for p in parts}) > 1:
                 parts = [p.to(torch.float32) for p in parts]
             return torch.stack(parts).contiguous()
 
-        self.gate, self.up, self.down = stack("gate"), stack("up"), stack("down")
+        self.gate = stack("gate", True) if self.gated else None
+        self.up, self.down = stack("up", True), stack("down", False)
 
     def forward(self, ctx: StepContext, h: torch.Tensor, residual: Optional[torch.Tensor]):
         T = h.shape[0]
-        logits = ctx.scratch("moe.logits", (T, self.outputs), torch.float32)
+        slots, real = self.top + self.shared_pieces, self.experts + self.shared_pieces
+        logits = ctx.scratch("moe.logits", (T, self.router.total_out), torch.float32)
         self.router(h, logits, ctx=ctx)
-        ids = ctx.scratch("moe.ids", (T, self.top), torch.int32)
-        weights = ctx.scratch("moe.weights", (T, self.top), torch.float32)
-        kernels.moe_route(logits, self.correction, self.groups, self.keep_groups, self.top, ids, weights)
-        tile_rows = kernels.moe_tile_rows(h.dtype, self.gate.dtype, self.hidden, self.intermediate, T * self.top,
-                                          self.experts)
-        rows = kernels.moe_align(ids, self.experts, tile_rows, ctx.scratch)
-        act = ctx.scratch("moe.act", (T * self.top, self.intermediate))
+        ids = ctx.scratch("moe.ids", (T, slots), torch.int32)
+        weights = ctx.scratch("moe.weights", (T, slots), torch.float32)
+        kernels.moe_route(logits, self.correction, self.groups, self.keep_groups, self.top, ids, weights,
+                          scoring=self.scoring, group_top=self.group_top, renormalize=self.renormalize,
+                          renorm_eps=self.renorm_eps, weight_scale=self.weight_scale, shared=self.shared_pieces)
+        tile_rows = kernels.moe_tile_rows(h.dtype, self.up.dtype, self.hidden, self.intermediate, T * slots, real)
+        rows = kernels.moe_align(ids, real, tile_rows, ctx.scratch)
+        act = ctx.scratch("moe.act", (T * slots, self.intermediate))
         kernels.moe_gate_up(h, self.gate, self.up, rows, act)
-        parts = ctx.scratch("moe.parts", (T * self.top, self.hidden), torch.float32)
+        parts = ctx.scratch("moe.parts", (T * slots, self.hidden), torch.float32)
         kernels.moe_down(act, self.down, rows, parts)
         routed = kernels.RoutedParts(parts, rows.where, weights, h)
         if residual is None:

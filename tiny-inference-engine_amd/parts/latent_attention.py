@@ -1,6 +1,7 @@
 """Attention over a cached latent: a token leaves one small vector and one rotated key part for all heads.
 
-    q = Wq h              per head [dim unrotated | rot_dim rotated]
+    q = Wq h              per head [dim unrotated | rot_dim rotated]; or, with ``q_rank``, through a latent of their
+                          own: c_q = RMSnorm(Wdq h) (weight ``dq_norm``), q = Wuq c_q
     Wdkv h                [kv_rank | rot_dim]: the first part RMS-normed (weight ``dkv_norm``) is the latent c, the
                           second, rotated by position, is the one rotated key part all heads share
     head h:  key = [Wuk[h] c | rotated part],  value = Wuv[h] c
@@ -18,7 +19,8 @@ kernels are the ones every other attention here uses. Prompt portions and decode
 Parameters: ``hidden``, ``num_heads``, ``head_dim`` (unrotated), ``rope_dim``, ``value_dim``, ``kv_rank``, ``scale``,
 ``window`` (None: all keys), ``sink`` (tensor name or None), ``eps``, ``position`` (a PartSpec of the position family
 that describes a rotation table over ``rope_dim``), ``names`` (``q``, ``dkv``, ``dkv_norm``, ``uk``, ``uv``, ``o`` and
-optionally ``g``), ``output_scale`` (a factor on the result, folded into the latent-to-value matrices).
+optionally ``g``; with ``q_rank`` ``dq``, ``dq_norm`` and ``uq`` instead of ``q``), ``output_scale`` (a factor on the
+result, folded into the latent-to-value matrices).
 """
 
 from __future__ import annotations
@@ -62,9 +64,14 @@ class LatentAttention(Mixer):
         self.q_width = H * (self.dim + self.rope_dim)
         self.latent_width = self.kv_rank + self.rope_dim
         self.gated = bool(names.get("g"))
-        inputs = [names["q"], names["dkv"]] + ([names["g"]] if self.gated else [])
-        sizes = [self.q_width, self.latent_width] + ([H * self.value_dim] if self.gated else [])
+        self.q_rank = int(params.get("q_rank") or 0)
+        first, first_width = (names["dq"], self.q_rank) if self.q_rank else (names["q"], self.q_width)
+        self.first_width = first_width
+        inputs = [first, names["dkv"]] + ([names["g"]] if self.gated else [])
+        sizes = [first_width, self.latent_width] + ([H * self.value_dim] if self.gated else [])
         self.inputs = Linear(inputs, sizes, self.hidden)
+        self.q_up = Linear([names["uq"]], [self.q_width], self.q_rank) if self.q_rank else None
+        self.q_norm: torch.Tensor = None
         self.out = Linear([names["o"]], [self.hidden], H * self.value_dim)
         self.position = build_part("position", params.get("position") or PartSpec("none"))
         table = self.position.rotary_table()
@@ -87,6 +94,9 @@ class LatentAttention(Mixer):
     def tensors(self) -> List[TensorSpec]:
         H, n = self.num_heads, self.names
         specs = self.inputs.tensors() + self.out.tensors()
+        if self.q_rank:
+            specs += self.q_up.tensors()
+            specs.append(TensorSpec(n["dq_norm"], (self.q_rank,), "vector", ("one_plus_uniform", 0.1)))
         specs.append(TensorSpec(n["dkv_norm"], (self.kv_rank,), "vector", ("one_plus_uniform", 0.1)))
         specs.append(TensorSpec(n["uk"], (H * self.dim, self.kv_rank), "matrix", ("normal", 0.05)))
         specs.append(TensorSpec(n["uv"], (H * self.value_dim, self.kv_rank), "matrix", ("normal", 0.05)))
@@ -99,6 +109,9 @@ class LatentAttention(Mixer):
         self.inputs.load(fetch)
         self.out.load(fetch)
         self.latent_norm = fetch(self.names["dkv_norm"], "vector")
+        if self.q_rank:
+            self.q_up.load(fetch)
+            self.q_norm = fetch(self.names["dq_norm"], "vector")
         uk = fetch(self.names["uk"], "matrix")
         self.uk_t = uk.view(H, self.dim, self.kv_rank).transpose(1, 2).contiguous()
         uv = fetch(self.names["uv"], "matrix").view(H, self.value_dim, self.kv_rank)
@@ -115,17 +128,26 @@ class LatentAttention(Mixer):
         q_plain = ctx.scratch("latent.q_plain", (T, H * self.dim))
         q_latent = ctx.scratch("latent.q", (T, H * D))
         step = cache.step
-        kernels.latent_prepare(proj, self.latent_norm, self.eps,
+        queries, latent_rows = proj, None
+        if self.q_rank:
+            # the queries' own latent: normed out of the first columns, then taken up to the heads
+            c_q = ctx.scratch("latent.c_q", (T, self.q_rank))
+            ctx.set_row_scale(c_q, None)
+            kernels.rms_norm_columns(proj[:, :self.q_rank], self.q_norm, self.eps, c_q)
+            queries = ctx.scratch("latent.queries", (T, self.q_width), torch.float32)
+            self.q_up(c_q, queries, ctx=ctx)
+            latent_rows = proj[:, self.q_rank:]
+        kernels.latent_prepare(queries, self.latent_norm, self.eps,
                                self.position.angles(ctx) if self.rotary_dim else None, self.rotary_dim, self.pairing,
                                step.slot_mapping, cache.k_cache, cache.v_cache, cache.block_size, cache.writes,
-                               q_plain, q_latent, H, self.dim, self.rope_dim, self.kv_rank)
+                               q_plain, q_latent, H, self.dim, self.rope_dim, self.kv_rank, latent_rows=latent_rows)
         q_heads = q_latent.view(T, H, D)
         kernels.head_linear(q_plain.view(T, H, self.dim), self.uk_t, q_heads[:, :, :self.kv_rank])
         attn = ctx.scratch("latent.attended", (T, H * D))
         kernels.paged_attention(q_latent, cache.k_cache, cache.v_cache, attn, step, ctx.batch, H, self.scale,
                                 self.window, scratch=ctx.scratch, sinks=self.sinks)
         heads = ctx.scratch("latent.heads", (T, H * self.value_dim))
-        gate = proj[:, self.q_width + self.latent_width:].unflatten(1, (H, self.value_dim)) if self.gated else None
+        gate = proj[:, self.first_width + self.latent_width:].unflatten(1, (H, self.value_dim)) if self.gated else None
         kernels.head_linear(attn.view(T, H, D)[:, :, :self.kv_rank], self.uv, heads.view(T, H, self.value_dim), gate)
         if residual is not None:
             self.out(heads, residual, accumulate=True, ctx=ctx)

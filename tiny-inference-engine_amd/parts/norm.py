@@ -10,6 +10,10 @@ would see anyway).
 ``layer_norm`` subtracts the row's mean first: ``out = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w``, a weight and
 no bias, statistics in float32. Parameters: ``dim``, ``eps``, ``weight``.
 
+``dynamic_tanh`` computes no mean and no variance: ``out = tanh(alpha * x) * w + b`` element by element, with the
+scalar ``alpha`` and the vectors ``w`` and ``b`` stored. It has an eps in no formula. Parameters: ``dim``, ``weight``,
+``bias``, ``alpha`` (tensor names).
+
 ``add_normed`` is the norm applied to a sub-layer's OUTPUT on its way into the stream, for arrangements that norm
 both sides of a sub-layer: ``x += RMSNorm(y) * w``, optionally with the next norm of the stream in the same pass.
 """
@@ -113,4 +117,43 @@ class LayerNorm(Norm):
         out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
         ctx.set_row_scale(out, None)
         kernels.layer_norm(x, self.weight, self.eps, out, rows)
+        return out
+
+
+@register_part("norm", "dynamic_tanh")
+class DynamicTanh(Norm):
+    capturable = True
+    replayable = True
+    adds_owed = True       # the pass that reads the stream adds the partial sums still owed to it
+
+    def __init__(self, params):
+        super().__init__(params)
+        self.dim = int(params["dim"])
+        self.weight_name = params["weight"]
+        self.bias_name = params["bias"]
+        self.alpha_name = params["alpha"]
+        self.weight: torch.Tensor = None
+        self.bias: torch.Tensor = None
+        self.alpha: torch.Tensor = None
+
+    def tensors(self) -> List[TensorSpec]:
+        return [TensorSpec(self.weight_name, (self.dim,), "vector", ("one_plus_uniform", 0.1)),
+                TensorSpec(self.bias_name, (self.dim,), "vector", ("normal", 0.05)),
+                TensorSpec(self.alpha_name, (1,), "vector", ("one_plus_uniform", 0.5))]   # a stored scalar reads as [1]
+
+    def load(self, fetch, mode, device) -> None:
+        self.weight = fetch(self.weight_name, "vector")
+        self.bias = fetch(self.bias_name, "vector")
+        self.alpha = fetch(self.alpha_name, "vector").reshape(1).contiguous()
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                out_name: str = "norm.out", out_dtype: torch.dtype = None) -> torch.Tensor:
+        count = x.shape[0] if rows is None else rows.numel()
+        out = ctx.scratch(out_name, (count, self.dim), out_dtype or ctx.act_dtype)
+        ctx.set_row_scale(out, None)
+        owed = ctx.take_owed(x)
+        if owed is not None and rows is not None:
+            kernels.add_partials(x, owed)
+            owed = None
+        kernels.dynamic_tanh(x, self.alpha, self.weight, self.bias, out, rows, owed)
         return out

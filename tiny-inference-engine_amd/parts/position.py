@@ -19,6 +19,12 @@ rotate, dimension i paired with i + r/2 and ``inv_freq[i] = theta^(-2i / r)``, t
 and both the cosine and the sine are multiplied by ``0.1 ln(factor) + 1``. Without ``scaling`` it is the plain
 rotation. ``pairing`` says which dimensions form a pair: ``rotate_half`` (i, i + r/2) or ``interleaved`` (2i, 2i + 1).
 Parameters: ``head_dim``, ``theta``, ``rotary_dim``, ``pairing``, ``scaling``.
+
+``rope_banded`` scales the frequencies by bands of wavelength: with ``f_i = theta^(-2i / r)``, wavelength
+``L_i = 2 pi / f_i`` and ``scaling`` = (factor, low, high, original), a pair keeps ``f_i`` where
+``L_i < original / high``, turns with ``f_i / factor`` where ``L_i > original / low``, and in between, with
+``s = (original / L_i - low) / (high - low)``, with ``(1 - s) f_i / factor + s f_i``. Amplitudes stay 1. Without
+``scaling`` it is the plain rotation. Parameters as for ``rope_yarn``.
 """
 
 from __future__ import annotations
@@ -148,5 +154,44 @@ class RopeYarn(Position):
         if table is None:
             table = ctx.scratch("rope.angles:" + repr(key), (ctx.num_tokens, self.rotary_dim), torch.float32)
             kernels.rope_angles(ctx.batch.positions, self.inv_freq, table, self.amplitude)
+            ctx.notes[key] = table
+        return table
+
+
+@register_part("position", "rope_banded")
+class RopeBanded(RopeYarn):
+    """A rotation whose long wavelengths are stretched by a factor, short ones kept, with a linear blend between."""
+
+    def __init__(self, params):
+        scaling = dict(params["scaling"]) if params.get("scaling") else None
+        super().__init__({**params, "scaling": None})
+        self.scaling = scaling
+        if scaling is not None:
+            for key in ("factor", "low", "high", "original"):
+                if not float(scaling[key]) > 0:
+                    raise InvalidArgument(f"rope scaling {key} must be positive, got {scaling[key]}")
+            if float(scaling["high"]) == float(scaling["low"]):
+                raise InvalidArgument("rope scaling needs 'high' and 'low' to differ")
+
+    def host_inv_freq(self) -> np.ndarray:
+        r = self.rotary_dim
+        i = np.arange(r // 2, dtype=np.float64)
+        freq = np.power(self.theta, -2.0 * i / r)
+        if self.scaling is not None:
+            factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+            low, high = float(self.scaling["low"]), float(self.scaling["high"])
+            wavelength = 2.0 * math.pi / freq
+            blend = (original / wavelength - low) / (high - low)
+            between = (1.0 - blend) * freq / factor + blend * freq
+            freq = np.where(wavelength < original / high, freq,
+                            np.where(wavelength > original / low, freq / factor, between))
+        return freq.astype(np.float32)
+
+    def angles(self, ctx) -> torch.Tensor:
+        key = ("rope_banded", self.rotary_dim, self.theta, repr(sorted((self.scaling or {}).items())))
+        table = ctx.notes.get(key)
+        if table is None:
+            table = ctx.scratch("rope.angles:" + repr(key), (ctx.num_tokens, self.rotary_dim), torch.float32)
+            kernels.rope_angles(ctx.batch.positions, self.inv_freq, table, 1.0)
             ctx.notes[key] = table
         return table
