@@ -4,7 +4,7 @@
     python bench.py --shape 32b                 the same measurements at the Qwen3-32B sizes
     python bench.py --sweep [--shape 32b]       decode at contexts 4096 / 16384 / 32768 x batch 1 / 8 / 32, a line a point
     python bench.py --workload stress           64 requests through the scheduler at the Qwen3-1.7B sizes
-    python bench.py --workload minerax          another design beside Qwen3 at equal sizes (also duzozen, topapel): prefill, decode
+    python bench.py --workload minerax          another design beside Qwen3 at equal sizes (also duzozen, topapel, zovudra): prefill, decode
 
 Prints ONE JSON line. A "step" is one decode step of the engine (schedule, build the batch, run
 the model, sample greedily) at the default batch of 8 with every sequence near the benchmark
@@ -149,11 +149,53 @@ def qwen3_beside_minerax(size):
                 intermediate_size=size["ff"], vocab_size=size["vocab"])
 
 
+# ``--workload zovudra``: the Zovudra design at sizes that resemble a real model's layers, beside Qwen3 with the same
+# stream, as many heads of the same size and a gated feed-forward as wide as Zovudra's dense ones. Layers repeat (an
+# attention with a window and four kept first positions and a dense feed-forward; the same with routed experts; a
+# latent attention whose cached head is 192 + 64 = 256 wide, with a dense feed-forward; attention with experts again);
+# every layer takes a per-token side input of 256. A token uses four routed experts of 768 and a shared one of 1536.
+ZOVUDRA_SIZES = {
+    "2k": {"width": 2048, "heads": 16, "kv_heads": 4, "dim": 128, "rot_dim": 64, "kv_rank": 192, "q_rank": 768,
+           "window": 1024, "keep_first": 4, "ff": 4096, "experts": 32, "expert_ff": 768, "top": 4, "shared_ff": 1536,
+           "side": 256, "layers": 8, "vocab": 32000},
+    "4k": {"width": 4096, "heads": 32, "kv_heads": 8, "dim": 128, "rot_dim": 64, "kv_rank": 192, "q_rank": 1536,
+           "window": 2048, "keep_first": 4, "ff": 8192, "experts": 64, "expert_ff": 1536, "top": 4, "shared_ff": 3072,
+           "side": 256, "layers": 4, "vocab": 32000},
+}
+
+
+def zovudra_config(size):
+    dense = {"kind": "dense", "ff": size["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "shared": {"ff": size["shared_ff"]},
+           "router": {"experts": size["experts"], "top": size["top"], "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+                 "scale": size["dim"] ** -0.5, "mask": {"size": size["window"], "keep_first": size["keep_first"]},
+                 "rot": {"dims": size["dim"], "base": 500000.0,
+                         "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    latent = {"heads": size["heads"], "dim": size["dim"], "rot_dim": size["rot_dim"], "vdim": size["dim"],
+              "kv_rank": size["kv_rank"], "q_rank": size["q_rank"], "scale": (size["dim"] + size["rot_dim"]) ** -0.5,
+              "mask": {"size": size["window"]}, "rot": {"dims": size["rot_dim"], "base": 10000.0}}
+    pattern = [{"type": "attention", "mixer": attention, "mlp": dense},
+               {"type": "attention", "mixer": attention, "mlp": moe},
+               {"type": "latent_attention", "mixer": latent, "mlp": dense},
+               {"type": "attention", "mixer": attention, "mlp": moe}]
+    return {"architecture": "Zovudra", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": size["width"] ** 0.5}, "token_side": {"dim": size["side"]},
+            "layers": [pattern[i % len(pattern)] for i in range(size["layers"])]}
+
+
+def qwen3_beside_zovudra(size):
+    return dict(QWEN3_8B, num_hidden_layers=size["layers"], hidden_size=size["width"],
+                num_attention_heads=size["heads"], num_key_value_heads=size["kv_heads"], head_dim=size["dim"],
+                intermediate_size=size["ff"], vocab_size=size["vocab"])
+
+
 # design -> (sizes, its config at a size, Qwen3 at that size, the context a decode step may reach)
 DESIGNS = {
     "duzozen": (DUZOZEN_SIZES, duzozen_config, qwen3_beside, lambda size: 2 * size["window"]),
     "topapel": (TOPAPEL_SIZES, topapel_config, qwen3_beside_topapel, lambda size: 2 * size["chunk"]),
     "minerax": (MINERAX_SIZES, minerax_config, qwen3_beside_minerax, lambda size: 4 * size["window"]),
+    "zovudra": (ZOVUDRA_SIZES, zovudra_config, qwen3_beside_zovudra, lambda size: 4 * size["window"]),
 }
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
@@ -412,9 +454,9 @@ def main():
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the shape has (0 = all)")
     parser.add_argument("--shape", choices=sorted(SHAPES), default=None,
                         help="layer sizes: 8b (default), 32b, or 1.7b (the default of --workload stress)")
-    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen", "topapel", "minerax"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "stress", "long-prompt", "duzozen", "topapel", "minerax", "zovudra"], default="decode",
                         help="decode: the headline measurement; stress: many requests through a small cache; "
-                             "long-prompt: one long prompt in portions; duzozen, topapel, minerax: that design beside Qwen3 at "
+                             "long-prompt: one long prompt in portions; duzozen, topapel, minerax, zovudra: that design beside Qwen3 at "
                              "equal sizes (--sizes), prefill and decode")
     parser.add_argument("--design-models", default="design,qwen3",
                         help="duzozen, topapel, minerax: which of the two models to run (design: the workload's own; or its name)")

@@ -137,7 +137,7 @@ def attend(q, keys, values, new, bs, dtype, window, keep, scale, H, free_passed_
             table[page] = -1
     step = SimpleNamespace(block_tables=i32([table + [0] * 3]), key_shares=None)
     batch = SimpleNamespace(query_start=i32([0, new]), context_lens=i32([T]), seq_of_row=i32([0] * new),
-                            all_decode=new == 1, num_seqs=1, plan_context=1024, host_new_tokens=[new],
+                            all_decode=new == 1, num_seqs=1, plan_context=max(1024, T), host_new_tokens=[new],
                             host_context_lens=[T], memo={}, num_tokens=new)
     qd = q[T - new:].reshape(new, H * D).to(dtype).cuda().contiguous()
     out = torch.empty_like(qd)
@@ -173,6 +173,26 @@ def test_a_window_beside_kept_first_positions(H, KVH, D, bs, window, keep, new, 
     want = plain_attend(q, keys, values, window, keep, 0.2, H)[T - new:]
     got = attend(q, keys, values, new, bs, dtype, window, keep, 0.2, H)
     close(got, want, 2e-5 if dtype == torch.float32 else 1.5e-2, f"attention, the last {new} rows")
+
+
+@pytest.mark.parametrize("new", [1, 3, 70])
+@pytest.mark.parametrize("H,KVH,D,bs,window,keep", [(8, 2, 64, 16, 1500, 70), (4, 4, 128, 16, 2000, 5), (4, 1, 48, 32, 900, 129)])
+def test_kept_positions_where_the_keys_are_cut_into_shares(H, KVH, D, bs, window, keep, new):
+    """A long context and few rows: the matrix-core kernels cut a row's keys into shares that are merged; the kept
+    keys go with the first share."""
+    from tie_amd import kernels
+
+    T = 2600
+    assert kernels.decode_splits(1, KVH, T, bs) > 1
+    q, keys, values = rnd(T, H, D, seed=1, scale=1.5), rnd(T, KVH, D, seed=2), rnd(T, KVH, D, seed=3)
+    for h in range(H):                       # the last query leans towards a kept key, so that losing it would show
+        q[T - 1, h] += 3.0 * keys[keep - 1, h // (H // KVH)]
+    q, keys, values = (t.to(torch.bfloat16).float() for t in (q, keys, values))
+    want = plain_attend(q, keys, values, window, keep, 0.2, H)[T - new:]
+    lost = plain_attend(q, keys, values, window, keep - 1, 0.2, H)[T - new:]
+    assert float((want - lost).abs().max()) > 0.05
+    got = attend(q, keys, values, new, bs, torch.bfloat16, window, keep, 0.2, H)
+    close(got, want, 1.5e-2, f"attention over shares, the last {new} rows")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -135,14 +135,17 @@ __device__ __forceinline__ void store_share(const floatx4 (&acc)[DTILES], float 
 // of the tile. The scores a lane then holds (rows quad * 4 + v of both sub-tiles) are those of the 8
 // consecutive keys quad * 8 .. + 7, which is also how the values of one dimension lie in a page: with
 // WIDE (block sizes in steps of 8) a lane reads them in one 16-byte piece.
-template <bool WIDE, bool CAPPED>
+// KEEPS: beside a window the keys of positions below `keep` are read as well, at their true positions. The wave
+// of the first share walks those the window has left behind, [0, min(keep, start)), tile by tile before its own
+// tiles, with addresses clamped into that range (the pages between it and the window may be gone).
+template <bool WIDE, bool CAPPED, bool KEEPS = false>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
     int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, int keep) {
   const int lane = threadIdx.x;
   const int col = lane & 15;   // query head within the group (column of every tile)
   const int quad = lane >> 4;  // 0..3
@@ -191,17 +194,18 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
 
   // Pages first, one tile further ahead than the data, so that no data load waits for a lookup.
   struct Pages { int k[2]; int v[WIDE ? 1 : 2]; };
-  auto lookup = [&](int base, Pages& pg) {
+  auto lookup_in = [&](int base, Pages& pg, int lo, int hi) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) pg.k[u] = table[page_of(min(max(base + krow0 + u * 4, start), pos))];
+    for (int u = 0; u < 2; ++u) pg.k[u] = table[page_of(min(max(base + krow0 + u * 4, lo), hi))];
 #pragma unroll
     for (int j = 0; j < (WIDE ? 1 : 2); ++j)
-      pg.v[j] = table[page_of(min(max(base + quad * 8 + j * 4, start / VG * VG), pos / VG * VG))];
+      pg.v[j] = table[page_of(min(max(base + quad * 8 + j * 4, lo / VG * VG), hi / VG * VG))];
   };
-  auto load_keys = [&](int base, const Pages& pg, u32x4_t (&kf)[2][KSTEPS]) {
+  auto lookup = [&](int base, Pages& pg) { lookup_in(base, pg, start, pos); };
+  auto load_keys_in = [&](int base, const Pages& pg, u32x4_t (&kf)[2][KSTEPS], int lo, int hi) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int kp = min(max(base + krow0 + u * 4, start), pos);
+      const int kp = min(max(base + krow0 + u * 4, lo), hi);
       const bf16_t* kr = k_cache + static_cast<size_t>(pg.k[u]) * page_stride + head_off +
                          static_cast<size_t>(offset_of(kp)) * DH;
 #pragma unroll
@@ -211,11 +215,12 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
       }
     }
   };
-  auto load_values = [&](int base, const Pages& pg, u32x4_t (&vf)[DTILES]) {
+  auto load_keys = [&](int base, const Pages& pg, u32x4_t (&kf)[2][KSTEPS]) { load_keys_in(base, pg, kf, start, pos); };
+  auto load_values_in = [&](int base, const Pages& pg, u32x4_t (&vf)[DTILES], int lo, int hi) {
     const bf16_t* vp[WIDE ? 1 : 2];
 #pragma unroll
     for (int j = 0; j < (WIDE ? 1 : 2); ++j) {
-      const int kp = min(max(base + quad * 8 + j * 4, start / VG * VG), pos / VG * VG);
+      const int kp = min(max(base + quad * 8 + j * 4, lo / VG * VG), hi / VG * VG);
       vp[j] = v_cache + static_cast<size_t>(pg.v[j]) * page_stride + head_off + offset_of(kp);
     }
 #pragma unroll
@@ -230,11 +235,23 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
       }
     }
   };
+  auto load_values = [&](int base, const Pages& pg, u32x4_t (&vf)[DTILES]) { load_values_in(base, pg, vf, start, pos); };
 
   // The loads of tile t + 1 are issued before the arithmetic of tile t, so memory latency and the
   // matrix cores overlap; the pages of tile t + 2 are looked up at the same time.
   u32x4_t kf[2][KSTEPS], vf[DTILES], kf_next[2][KSTEPS], vf_next[DTILES];
   Pages pages;
+  if constexpr (KEEPS) {
+    const int kept_last = min(keep, start) - 1;     // the kept keys before the window: 0 .. kept_last
+    if (split == 0) {
+      for (int base = 0; base <= kept_last; base += 32) {
+        lookup_in(base, pages, 0, kept_last);
+        load_keys_in(base, pages, kf, 0, kept_last);
+        load_values_in(base, pages, vf, 0, kept_last);
+        attend_tile<CAPPED>(kf, vf, qf, acc, m, l, base, 0, kept_last, quad, scale_log2e, cap);
+      }
+    }
+  }
   if (tile_begin < tile_end) {
     lookup(tile_begin * 32, pages);
     load_keys(tile_begin * 32, pages, kf_next);
@@ -292,7 +309,7 @@ struct QkSource {
   int write_kv;            // 0: the cache holds the newest token already (another layer's cache)
 };
 
-template <int DEPTH, bool PREPARE, bool CAPPED>
+template <int DEPTH, bool PREPARE, bool CAPPED, bool KEEPS = false>
 __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     const bf16_t* __restrict__ q, bf16_t* k_cache, bf16_t* v_cache,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -300,7 +317,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     const int* __restrict__ block_tables, const int* __restrict__ seq_ids, int H, int KVH, int block_size,
     int block_shift, int max_blocks, float scale_log2e, float cap, int window, int nsplit,
     const float* __restrict__ sinks, const int* __restrict__ share_tiles,
-    QkSource src) {
+    QkSource src, int keep) {
   const int lane = threadIdx.x;
   const int col = lane & 15;
   const int quad = lane >> 4;
@@ -370,14 +387,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
 
   struct Tile { u32x4_t k[2][KSTEPS]; u32x4_t v[DTILES]; };
   // Positions are clamped into [start, pos] for addresses only; a clamped position stays in its half of 16.
-  auto issue = [&](int tile, Tile& tl) {
+  auto issue_in = [&](int tile, Tile& tl, int lo, int hi) {
     const int base = tile * 32;
-    const int page_lo = table[min(max(base, start), pos) >> block_shift];
-    const int page_hi = table[min(max(base + 16, start), pos) >> block_shift];
+    const int page_lo = table[min(max(base, lo), hi) >> block_shift];
+    const int page_hi = table[min(max(base + 16, lo), hi) >> block_shift];
     const bf16_t* kpage = k_cache + static_cast<size_t>(keys_in_upper_half ? page_hi : page_lo) * page_stride + head_off;
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
-      const int kp = min(max(base + krow0 + u * 4, start), pos);
+      const int kp = min(max(base + krow0 + u * 4, lo), hi);
       const bf16_t* kr = kpage + static_cast<size_t>(kp & in_page) * DH;
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st) {
@@ -390,13 +407,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
         tl.k[u][st] = inside ? piece : u32x4_t{0, 0, 0, 0};
       }
     }
-    const int vp = min(max(base + quad * 8, start / 8 * 8), pos / 8 * 8);
+    const int vp = min(max(base + quad * 8, lo / 8 * 8), hi / 8 * 8);
     const bf16_t* vr = v_cache + static_cast<size_t>(values_in_upper_half ? page_hi : page_lo) * page_stride + head_off +
                        (vp & in_page) + dim_off;
 #pragma unroll
     for (int dt = 0; dt < DTILES; ++dt)
       tl.v[dt] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(vr + static_cast<size_t>(dt) * 16 * block_size));
   };
+  auto issue = [&](int tile, Tile& tl) { issue_in(tile, tl, start, pos); };
 
   // Tile i of the wave lives in set i % DEPTH. The groups of DEPTH tiles in the middle issue and compute
   // without a condition, so the compiler knows how many loads are in flight and waits for the oldest tile
@@ -479,6 +497,18 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
       qf[st] = (col < G && d < DH) ? *reinterpret_cast<const u32x4_t*>(q_lds + col * DH + d) : u32x4_t{0, 0, 0, 0};
     }
   }
+  if constexpr (KEEPS) {
+    // The kept keys the window has left behind, by the first share's wave, through the ring's last set (the
+    // first tiles' loads are on their way in the others).
+    const int kept_last = min(keep, start) - 1;
+    if (split == 0) {
+      for (int kt = 0; kt * 32 <= kept_last; ++kt) {
+        issue_in(kt, ring[DEPTH - 1], 0, kept_last);
+        attend_tile<CAPPED>(ring[DEPTH - 1].k, ring[DEPTH - 1].v, qf, acc, m, l, kt * 32, 0, kept_last, quad,
+                            scale_log2e, cap);
+      }
+    }
+  }
   int tile = tile_begin;
   for (; tile + 2 * DEPTH - 2 < tile_end; tile += DEPTH) {
 #pragma unroll
@@ -552,7 +582,9 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
                          float* part_o, float* part_ml, const int* query_start, const int* context_lens,
                          const int* block_tables, const int* seq_ids, int num_seqs, int H, int KVH, int block_size,
                          int max_blocks, float scale, float softcap, int window, int nsplit, const int* share_tiles,
-                         int depth, const float* sinks, hipStream_t stream) {
+                         int depth, const float* sinks, hipStream_t stream, int keep = 0) {
+  // kept first positions go beside a window, with uncapped scores and queries that come ready
+  if (keep < 0 || (keep > 0 && (window <= 0 || softcap > 0.f || src != nullptr))) return TIE_BAD_ARGUMENT;
   if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
@@ -573,21 +605,26 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   // Capped scores are an instantiation of their own: the uncapped kernels carry none of it.
 #define LAUNCH_RING(DEPTH)                                                                                   \
   {                                                                                                          \
-    if (src == nullptr && cap > 0.f) {                                                                       \
+    if (keep > 0) {                                                                                          \
+      attention_decode_ring_kernel<DEPTH, false, false, true><<<grid, TIE_WAVE, 0, stream>>>(                \
+          q, k_cache, v_cache, ARGS, share_tiles, QkSource{}, keep);                                         \
+    } else if (src == nullptr && cap > 0.f) {                                                                \
       attention_decode_ring_kernel<DEPTH, false, true><<<grid, TIE_WAVE, 0, stream>>>(                       \
-          q, k_cache, v_cache, ARGS, share_tiles, QkSource{});                                               \
+          q, k_cache, v_cache, ARGS, share_tiles, QkSource{}, 0);                                            \
     } else if (src == nullptr) {                                                                             \
       attention_decode_ring_kernel<DEPTH, false, false><<<grid, TIE_WAVE, 0, stream>>>(                      \
-          q, k_cache, v_cache, ARGS, share_tiles, QkSource{});                                               \
+          q, k_cache, v_cache, ARGS, share_tiles, QkSource{}, 0);                                            \
     } else if constexpr (PREPARE_HEAD_DIM) {                                                                 \
       attention_decode_ring_kernel<DEPTH, true, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache,   \
-                                                                                      ARGS, share_tiles, *src); \
+                                                                                      ARGS, share_tiles, *src, 0); \
     }                                                                                                        \
   }
 #define LAUNCH_PLAIN(WIDE)                                                                                   \
   {                                                                                                          \
-    if (cap > 0.f) attention_decode_kernel<WIDE, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS); \
-    else attention_decode_kernel<WIDE, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS);     \
+    if (keep > 0)                                                                                            \
+      attention_decode_kernel<WIDE, false, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS, keep); \
+    else if (cap > 0.f) attention_decode_kernel<WIDE, true><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS, 0); \
+    else attention_decode_kernel<WIDE, false><<<grid, TIE_WAVE, 0, stream>>>(q, k_cache, v_cache, ARGS, 0);  \
   }
   if (src != nullptr && cap > 0.f) return TIE_BAD_ARGUMENT;   // the kernel that makes its own queries caps nothing
   if (depth == 4) LAUNCH_RING(4)
@@ -610,6 +647,22 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
 // much (the ring kernel and more than one share only; 0 there means shares by each sequence's own length).
 // chunk > 0 (then window must be 0): a query reads the keys of its own chunk of that many positions, counted from
 // position 0. sinks (or null): one float a query head whose exponential joins the head's softmax denominator.
+// keep > 0 (beside a window, with uncapped scores): the keys of positions below keep are read as well.
+extern "C" int tie_attention_decode_bf16_keeping(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                                 float* part_o, float* part_ml, const int* query_start,
+                                                 const int* context_lens, const int* block_tables, const int* seq_ids,
+                                                 int num_seqs, int H, int KVH, int block_size, int max_blocks,
+                                                 float scale, float softcap, int window, int nsplit,
+                                                 const int* share_tiles, int depth, int chunk, const float* sinks,
+                                                 int keep, hipStream_t stream) {
+  if (window < 0 || chunk < 0 || (window > 0 && chunk > 0)) return TIE_BAD_ARGUMENT;
+  if (chunk > 0) window = -chunk;
+  return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
+                       static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
+                       query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
+                       scale, softcap, window, nsplit, share_tiles, depth, sinks, stream, keep);
+}
+
 extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
                                               float* part_o, float* part_ml, const int* query_start,
                                               const int* context_lens, const int* block_tables, const int* seq_ids,
@@ -617,12 +670,9 @@ extern "C" int tie_attention_decode_bf16_with(const void* q, const void* k_cache
                                               float scale, float softcap, int window, int nsplit,
                                               const int* share_tiles, int depth, int chunk, const float* sinks,
                                               hipStream_t stream) {
-  if (window < 0 || chunk < 0 || (window > 0 && chunk > 0)) return TIE_BAD_ARGUMENT;
-  if (chunk > 0) window = -chunk;
-  return launch_decode(static_cast<const bf16_t*>(q), nullptr, static_cast<bf16_t*>(const_cast<void*>(k_cache)),
-                       static_cast<bf16_t*>(const_cast<void*>(v_cache)), static_cast<bf16_t*>(out), part_o, part_ml,
-                       query_start, context_lens, block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks,
-                       scale, softcap, window, nsplit, share_tiles, depth, sinks, stream);
+  return tie_attention_decode_bf16_keeping(q, k_cache, v_cache, out, part_o, part_ml, query_start, context_lens,
+                                           block_tables, seq_ids, num_seqs, H, KVH, block_size, max_blocks, scale,
+                                           softcap, window, nsplit, share_tiles, depth, chunk, sinks, 0, stream);
 }
 
 // The same for a step of single decoded tokens whose queries, newest keys and values still lie in the QKV

@@ -152,13 +152,17 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16
 
 // items: [num_items][2] = (sequence, index of its first new row handled here); the last items run first.
 // WIDE: the block size is a multiple of 8, so 8 keys of one value dimension lie together in a page.
-template <int HC, int QC, bool WIDE, bool CAPPED>
+// KEEPS: beside a window the keys of positions below `keep` are read as well, at their true positions. The
+// workgroup of an item's first share walks those that lie before the window of its last row, tile by tile ahead of
+// its own tiles, through the first LDS buffer, with addresses clamped into that range (the pages between it and the
+// window may be gone); a row takes of them the keys before its own window, the others it meets among its own tiles.
+template <int HC, int QC, bool WIDE, bool CAPPED, bool KEEPS = false>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     bf16_t* __restrict__ out, const int* __restrict__ query_start, const int* __restrict__ context_lens,
     const int* __restrict__ block_tables, const int* __restrict__ items, int num_items, int H, int KVH, int block_size,
     int max_blocks, float scale_log2e, float cap, int window, int block_shift, int flip_from, int nsplit,
-    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, const float* __restrict__ sinks, int keep) {
   extern __shared__ __align__(16) unsigned char smem[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(smem);
   const int wave = threadIdx.x / TIE_WAVE;
@@ -232,6 +236,79 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const int first_v = wg_first / VG * VG, last_v = wg_last / VG * VG;
   u32x4_t kreg[K_PER_THREAD], vreg[V_PER_THREAD];
   int kpage[K_PER_THREAD], vpage[V_PER_THREAD][WIDE ? 1 : 2];
+  if constexpr (KEEPS) {
+    const int kept_end = min(keep, first_visible_key(wg_last, window));   // kept keys before the last row's window
+    if (split == 0 && kept_end > 0) {
+      const int kept_mine = min(keep, lo);                  // of them, those before this lane's row's own window
+      const int wg_first = 0, wg_last = kept_end - 1;       // the ranges the loading macros clamp into
+      const int first_v = 0, last_v = wg_last / VG * VG;
+      for (int kt = 0; kt * KT < kept_end; ++kt) {
+        LOAD_PAGES(kt);
+        LOAD_TILE(kt);
+        STORE_TILE(lds, lds + KT * KROW);
+        __syncthreads();
+        const bf16_t* k_lds = lds;
+        const bf16_t* v_lds = lds + KT * KROW;
+        const int base = kt * KT;
+        if (wave_active) {
+          floatx16 sc[2];
+          const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+              Frag a;
+              a.u4 = *reinterpret_cast<const uint4*>(k_lds + (u * 32 + r32) * KROW + ks * 16 + hi * 8);
+              sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[ks].v, ks == 0 ? zero : sc[u], 0, 0, 0);
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int kp = base + u * 32 + 8 * (v / 4) + hi * 4 + (v % 4);
+              sc[u][v] = kp < kept_mine ? sc[u][v] : -INFINITY;
+            }
+          float tile_max = -INFINITY;
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) tile_max = fmaxf(tile_max, sc[u][v]);
+          tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, TIE_WAVE));
+          const float m_new = fmaxf(m, tile_max);
+          const float neg_mc = (m_new == -INFINITY) ? 0.f : -m_new * scale_log2e;
+          const float corr = __builtin_amdgcn_exp2f(fmaf(m, scale_log2e, neg_mc));   // m = -inf: 0
+          Frag pf[4];
+          float psum = 0.f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[j / 2][(j % 2) * 8 + e], scale_log2e, neg_mc));
+              const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[j / 2][(j % 2) * 8 + e + 1], scale_log2e, neg_mc));
+              psum += p0;
+              psum += p1;
+              pf[j].w[e / 2] = pack2(p0, p1);
+            }
+          l = l * corr + psum;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[dt][v] *= corr;
+          m = m_new;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              Frag a;
+              a.u4 = *reinterpret_cast<const uint4*>(v_lds + (dt * 32 + r32) * VROW + j * 16 + hi * 8);
+              acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, pf[j].v, acc[dt], 0, 0, 0);
+            }
+        }
+        __syncthreads();                       // the buffer is written again by the next tile
+      }
+    }
+  }
   if (!empty) {
     LOAD_PAGES(tile_begin);
     LOAD_TILE(tile_begin);
@@ -702,12 +779,12 @@ static int launch_prefill_dma(const dim3 grid, hipStream_t stream, const bf16_t*
   return tie_launch_status();
 }
 
-template <int HC, int QC, bool WIDE, bool CAPPED>
+template <int HC, int QC, bool WIDE, bool CAPPED, bool KEEPS = false>
 static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_cache,
                           const bf16_t* v_cache, bf16_t* out, const int* query_start, const int* context_lens,
                           const int* block_tables, const int* items, int num_items, int H, int KVH, int block_size,
                           int max_blocks, float scale_log2e, float cap, int window, int nsplit, float* part_o, float* part_ml,
-                          const float* sinks) {
+                          const float* sinks, int keep = 0) {
   const int block_shift = __builtin_ctz(block_size);   // block sizes are powers of two here
   // One resident round (at most two workgroups on each of the compute units): see the kernel's item order.
   const long planes = static_cast<long>(grid.y) * grid.z;
@@ -716,14 +793,15 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
   constexpr size_t lds_bytes = 2 * static_cast<size_t>(LDS_TILE) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<HC, QC, WIDE, CAPPED>),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
+    const hipError_t e = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(&attention_prefill_kernel<HC, QC, WIDE, CAPPED, KEEPS>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes));
     if (e != hipSuccess) return static_cast<int>(e);
     configured = true;
   }
-  attention_prefill_kernel<HC, QC, WIDE, CAPPED><<<grid, THREADS, lds_bytes, stream>>>(
+  attention_prefill_kernel<HC, QC, WIDE, CAPPED, KEEPS><<<grid, THREADS, lds_bytes, stream>>>(
       q, k_cache, v_cache, out, query_start, context_lens, block_tables, items, num_items, H, KVH, block_size,
-      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml, sinks);
+      max_blocks, scale_log2e, cap, window, block_shift, flip_from, nsplit, part_o, part_ml, sinks, keep);
   return tie_launch_status();
 }
 
@@ -732,16 +810,20 @@ static int launch_prefill(const dim3 grid, hipStream_t stream, const bf16_t* q, 
 // partial results and a second kernel merges them into out for the num_rows rows of the step.
 // staging: 0 = by the rule, 1 = tiles copied through registers (any page size and head size), 2 = tiles loaded
 // straight into LDS (pages of 16 positions or more, head sizes 32, 64, 128, 256; refused otherwise).
-extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
-                                               const int* query_start, const int* context_lens,
-                                               const int* block_tables, const int* items, int num_items, int H,
-                                               int KVH, int block_size, int max_blocks, float scale, float softcap,
-                                               int window, int nsplit, float* part_o, float* part_ml,
-                                               const int* merge_rows, int num_merge_rows, int staging,
-                                               int chunk, const float* sinks, hipStream_t stream) {
+// keep > 0 (beside a window, with uncapped scores): the keys of positions below keep are read as well; such steps
+// copy their tiles through registers (staging 0 or 1).
+extern "C" int tie_attention_prefill_bf16_keeping(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                                  const int* query_start, const int* context_lens,
+                                                  const int* block_tables, const int* items, int num_items, int H,
+                                                  int KVH, int block_size, int max_blocks, float scale, float softcap,
+                                                  int window, int nsplit, float* part_o, float* part_ml,
+                                                  const int* merge_rows, int num_merge_rows, int staging,
+                                                  int chunk, const float* sinks, int keep, hipStream_t stream) {
   // chunk > 0 (then window must be 0): a query reads the keys of its own chunk of that many positions, counted
   // from position 0. sinks (or null): one float a query head whose exponential joins its softmax denominator.
   if (window < 0 || chunk < 0 || (window > 0 && chunk > 0)) return TIE_BAD_ARGUMENT;
+  if (keep < 0 || (keep > 0 && (window <= 0 || softcap > 0.f || staging == 2))) return TIE_BAD_ARGUMENT;
+  if (keep > 0) staging = 1;
   if (chunk > 0) window = -chunk;
   if (num_items <= 0 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || block_size < 4 ||
       (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || !(scale > 0.f) || nsplit < 1 ||
@@ -768,12 +850,16 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
       items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml, sinks)
 #define LAUNCH(HC, QC)                                                                                            \
-  status = (block_size % 8 == 0                                                                                   \
-                ? (cap > 0.f ? launch_prefill<HC, QC, true, true> : launch_prefill<HC, QC, true, false>)          \
-                : (cap > 0.f ? launch_prefill<HC, QC, false, true> : launch_prefill<HC, QC, false, false>))(      \
+  status = (keep > 0                                                                                              \
+                ? (block_size % 8 == 0 ? launch_prefill<HC, QC, true, false, true>                                \
+                                       : launch_prefill<HC, QC, false, false, true>)                              \
+                : block_size % 8 == 0                                                                             \
+                      ? (cap > 0.f ? launch_prefill<HC, QC, true, true> : launch_prefill<HC, QC, true, false>)    \
+                      : (cap > 0.f ? launch_prefill<HC, QC, false, true> : launch_prefill<HC, QC, false, false>))( \
       grid, stream, static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache),                           \
       static_cast<const bf16_t*>(v_cache), static_cast<bf16_t*>(out), query_start, context_lens, block_tables,    \
-      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml, sinks)
+      items, num_items, H, KVH, block_size, max_blocks, scale_log2e, cap, window, nsplit, part_o, part_ml, sinks, \
+      keep)
   if (dma) {
     if constexpr (DMA_HEAD_DIM) {
       if (hc == 4) LAUNCH_DMA(4, 1);
@@ -793,6 +879,19 @@ extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cach
   launch_attention_merge(part_o, part_ml, static_cast<bf16_t*>(out), merge_rows, nullptr, nullptr, H, nsplit,
                          num_merge_rows, sinks, stream);
   return tie_launch_status();
+}
+
+extern "C" int tie_attention_prefill_bf16_with(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                               const int* query_start, const int* context_lens,
+                                               const int* block_tables, const int* items, int num_items, int H,
+                                               int KVH, int block_size, int max_blocks, float scale, float softcap,
+                                               int window, int nsplit, float* part_o, float* part_ml,
+                                               const int* merge_rows, int num_merge_rows, int staging,
+                                               int chunk, const float* sinks, hipStream_t stream) {
+  return tie_attention_prefill_bf16_keeping(q, k_cache, v_cache, out, query_start, context_lens, block_tables, items,
+                                            num_items, H, KVH, block_size, max_blocks, scale, softcap, window, nsplit,
+                                            part_o, part_ml, merge_rows, num_merge_rows, staging, chunk, sinks, 0,
+                                            stream);
 }
 
 extern "C" int tie_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, void* out,

@@ -195,6 +195,10 @@ _SIGNATURES = {
         "tie_attention_prefill_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int,
                                             _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void, _c_void],
+        "tie_attention_prefill_bf16_keeping": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int,
+                                               _c_int, _c_void, _c_void, _c_void, _c_int, _c_int, _c_int, _c_void,
+                                               _c_int, _c_void],
     },
     "attention_decode_bf16": {
         "tie_attention_decode_head_dim": [],
@@ -210,6 +214,10 @@ _SIGNATURES = {
         "tie_attention_decode_bf16_with": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
                                            _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float,
                                            _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_void],
+        "tie_attention_decode_bf16_keeping": [_c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void, _c_void,
+                                              _c_void, _c_void, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                              _c_float, _c_int, _c_int, _c_void, _c_int, _c_int, _c_void, _c_int,
+                                              _c_void],
     },
 }
 
@@ -1328,11 +1336,13 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
                           seq_ids: Optional[torch.Tensor] = None, depth: int = 0,
                           share_tiles: Optional[torch.Tensor] = None, softcap: Optional[float] = None,
-                          chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> None:
+                          chunk: Optional[int] = None, sinks: Optional[torch.Tensor] = None,
+                          keep_first: int = 0) -> None:
     """Attention for sequences that bring one new row each (``seq_ids`` selects them; None = all).
 
     ``chunk`` n (instead of a ``window``): a query at position p reads the keys from ``p - p % n`` on. ``sinks``
-    (float32 ``[heads]``): ``exp(sinks[h])`` is one more term of head h's softmax denominator.
+    (float32 ``[heads]``): ``exp(sinks[h])`` is one more term of head h's softmax denominator. ``keep_first`` f
+    (beside a ``window``, with uncapped scores): the keys of positions below f are read as well.
 
     ``share_tiles`` (one int32 on the device, or None): the length of every share in tiles of 32 keys, for steps
     whose sequences differ much in length (``decode_share_plan``); with pages of 16 positions or more and more than
@@ -1374,11 +1384,13 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         _i32(share_tiles, "the shares' length", 1)
         if nsplit == 1 or bs < 16 or depth == 1:
             raise InvalidArgument("a length for all shares goes with more than one share and pages of 16 positions or more")
-    _call(lib.tie_attention_decode_bf16_with, "attention_decode_bf16",
+    if keep_first and (not window or softcap):
+        raise InvalidArgument("first positions are kept beside a sliding window, with uncapped scores")
+    _call(lib.tie_attention_decode_bf16_keeping, "attention_decode_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), _ptr(part_o), _ptr(part_ml),
         query_start.data_ptr(), context_lens.data_ptr(), block_tables.data_ptr(), _ptr(seq_ids), num_seqs, H, KVH, bs,
         block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), nsplit, _ptr(share_tiles), depth,
-        int(chunk or 0), _ptr(_sinks(sinks, H, window, chunk)), _stream())
+        int(chunk or 0), _ptr(_sinks(sinks, H, window, chunk)), int(keep_first or 0), _stream())
 
 
 def _sinks(sinks: Optional[torch.Tensor], heads: int, window, chunk) -> Optional[torch.Tensor]:
@@ -1465,8 +1477,11 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                            nsplit: int = 1, part_o: Optional[torch.Tensor] = None,
                            part_ml: Optional[torch.Tensor] = None, merge_rows: Optional[torch.Tensor] = None,
                            staging: int = 0, softcap: Optional[float] = None, chunk: Optional[int] = None,
-                           sinks: Optional[torch.Tensor] = None) -> None:
+                           sinks: Optional[torch.Tensor] = None, keep_first: int = 0) -> None:
     """Causal attention of the new rows of the sequences ``items`` names over their cached keys.
+
+    ``keep_first`` f (beside a ``window``, with uncapped scores): the keys of positions below f are read as well;
+    such steps copy their tiles through registers.
 
     ``staging`` picks how key tiles reach LDS: 1 = copied through registers (any page and head size),
     2 = loaded straight into LDS (``prefill_loads_straight``), 0 = the second where it applies.
@@ -1492,8 +1507,11 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
                               f"16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
     if staging not in (0, 1, 2) or (staging == 2 and not prefill_loads_straight(Dh, bs)):
         raise InvalidArgument(f"attention_prefill_bf16: staging {staging} with head_dim {Dh} and pages of {bs} positions")
+    if keep_first and (not window or softcap or staging == 2):
+        raise InvalidArgument("first positions are kept beside a sliding window, with uncapped scores and tiles copied "
+                              "through registers")
     if staging == 0:
-        staging = 2 if prefill_loads_straight(Dh, bs) else 1
+        staging = 2 if prefill_loads_straight(Dh, bs) and not keep_first else 1
     if staging == 1 and not prefill_addressable(k_cache):
         raise InvalidArgument(f"attention_prefill_bf16 addresses cache planes under 32 GB (pages under 128 MB, under 2^24 "
                               f"pages); got {NB} pages of {k_cache[0].numel() * k_cache.element_size()} bytes")
@@ -1513,12 +1531,12 @@ def attention_prefill_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
         if part_o.numel() < rows * H * nsplit * Dh or part_ml.numel() < rows * H * nsplit * 2 or not 0 < num_merge <= 65535:
             raise InvalidArgument("the buffers for the splits are too small, or no (or too many) rows to merge")
     lib = _lib("attention_prefill_bf16", Dh)
-    _call(lib.tie_attention_prefill_bf16_with, "attention_prefill_bf16",
+    _call(lib.tie_attention_prefill_bf16_keeping, "attention_prefill_bf16",
         q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), query_start.data_ptr(),
         context_lens.data_ptr(), block_tables.data_ptr(), items.data_ptr(), items.shape[0], H, KVH, bs,
         block_tables.shape[1], float(scale), float(softcap or 0.0), int(window or 0), int(nsplit), _ptr(part_o),
         _ptr(part_ml), _ptr(merge_rows), num_merge, staging, int(chunk or 0),
-        _ptr(_sinks(sinks, num_heads, window, chunk)), _stream())
+        _ptr(_sinks(sinks, num_heads, window, chunk)), int(keep_first or 0), _stream())
 
 
 def prefill_splits(num_items: int, num_kv_heads: int, group_size: int, max_context: int, num_rows: int) -> int:
@@ -1547,8 +1565,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             and num_heads % KVH == 0 and mfma_block_size(bs) and scratch is not None)
     if keep_first and not window:
         raise InvalidArgument("first positions are kept beside a sliding window only")
-    if keep_first:
-        fast = False           # kept first positions: the generic kernel walks them
+    if keep_first and softcap:
+        fast = False           # kept first positions beside capped scores: the generic kernel alone takes both
     reach = (window + keep_first if window else None) or chunk      # the most keys a query reads: what the shares of a sequence's keys are planned by
     if fast and batch.all_decode and num_heads // KVH <= 16:
         S = batch.num_seqs
@@ -1559,7 +1577,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             part_ml = scratch("attention.split_ml", (S * num_heads * nsplit * 2,), torch.float32)
         attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                               S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles,
-                              softcap=softcap, chunk=chunk, sinks=sinks)
+                              softcap=softcap, chunk=chunk, sinks=sinks, keep_first=keep_first)
         return
     if fast and batch.all_decode:
         # Single tokens of more than 16 query heads a KV head: the decode kernel does not take them, and the work
@@ -1606,8 +1624,9 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.split_ml", (num_single * num_heads * nsplit * 2,), torch.float32)
             attention_decode_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                                   num_single, num_heads, scale, window, nsplit, part_o, part_ml, seq_ids=seq_ids,
-                                  share_tiles=share_tiles, softcap=softcap, chunk=chunk, sinks=sinks)
-        if items is not None and not prefill_loads_straight(Dh, bs) and not prefill_addressable(k_cache):
+                                  share_tiles=share_tiles, softcap=softcap, chunk=chunk, sinks=sinks,
+                                  keep_first=keep_first)
+        if items is not None and (keep_first or not prefill_loads_straight(Dh, bs)) and not prefill_addressable(k_cache):
             # A cache plane the prefill kernel cannot address: the prompt portions go to the generic kernel
             # (which runs every row of the step; the single rows above are simply computed again).
             paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
@@ -1624,7 +1643,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                 part_ml = scratch("attention.prefill_split_ml", (rows * num_heads * nsplit * 2,), torch.float32)
             attention_prefill_bf16(q, k_cache, v_cache, out, batch.query_start, batch.context_lens,
                                    step.block_tables, items, num_heads, scale, window, nsplit, part_o, part_ml,
-                                   merge_rows if nsplit > 1 else None, softcap=softcap, chunk=chunk, sinks=sinks)
+                                   merge_rows if nsplit > 1 else None, softcap=softcap, chunk=chunk, sinks=sinks,
+                                   keep_first=keep_first)
         return
     paged_attention_generic(q, k_cache, v_cache, out, batch.query_start, batch.context_lens, step.block_tables,
                             batch.seq_of_row, num_heads, scale, window, softcap, chunk, sinks, keep_first)
