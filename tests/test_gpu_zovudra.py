@@ -176,10 +176,11 @@ def test_a_window_beside_kept_first_positions(H, KVH, D, bs, window, keep, new, 
 
 
 @pytest.mark.parametrize("new", [1, 3, 70])
-@pytest.mark.parametrize("H,KVH,D,bs,window,keep", [(8, 2, 64, 16, 1500, 70), (4, 4, 128, 16, 2000, 5), (4, 1, 48, 32, 900, 129)])
+@pytest.mark.parametrize("H,KVH,D,bs,window,keep", [(8, 2, 64, 16, 1500, 70), (4, 4, 128, 16, 2000, 5), (4, 1, 48, 32, 900, 129),
+                                                    (40, 2, 64, 16, 1200, 33), (17, 1, 128, 16, 2000, 0)])
 def test_kept_positions_where_the_keys_are_cut_into_shares(H, KVH, D, bs, window, keep, new):
     """A long context and few rows: the matrix-core kernels cut a row's keys into shares that are merged; the kept
-    keys go with the first share."""
+    keys go with the first share. More than sixteen query heads on a key/value head are several waves of columns."""
     from tie_amd import kernels
 
     T = 2600
@@ -189,8 +190,9 @@ def test_kept_positions_where_the_keys_are_cut_into_shares(H, KVH, D, bs, window
         q[T - 1, h] += 3.0 * keys[keep - 1, h // (H // KVH)]
     q, keys, values = (t.to(torch.bfloat16).float() for t in (q, keys, values))
     want = plain_attend(q, keys, values, window, keep, 0.2, H)[T - new:]
-    lost = plain_attend(q, keys, values, window, keep - 1, 0.2, H)[T - new:]
-    assert float((want - lost).abs().max()) > 0.05
+    if keep:
+        lost = plain_attend(q, keys, values, window, keep - 1, 0.2, H)[T - new:]
+        assert float((want - lost).abs().max()) > 0.05
     got = attend(q, keys, values, new, bs, torch.bfloat16, window, keep, 0.2, H)
     close(got, want, 1.5e-2, f"attention over shares, the last {new} rows")
 

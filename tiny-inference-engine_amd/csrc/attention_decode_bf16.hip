@@ -150,9 +150,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   const int col = lane & 15;   // query head within the group (column of every tile)
   const int quad = lane >> 4;  // 0..3
   const int split = blockIdx.x;
-  const int kvh = blockIdx.y;
+  // More than 16 query heads a KV head run as several waves of up to 16 columns each: blockIdx.y counts
+  // (KV head, group of 16 heads).
+  const int heads_per_kv = H / KVH;
+  const int column_groups = (heads_per_kv + 15) / 16;
+  const int kvh = static_cast<int>(blockIdx.y) / column_groups;
+  const int head0 = kvh * heads_per_kv + (static_cast<int>(blockIdx.y) % column_groups) * 16;   // column 0's query head
   const int s = seq_ids ? seq_ids[blockIdx.z] : blockIdx.z;
-  const int G = H / KVH;
+  const int G = min(16, kvh * heads_per_kv + heads_per_kv - head0);                          // this wave's columns
   const int t = query_start[s];            // the sequence's single new row
   const int pos = context_lens[s] - 1;     // its position; keys start..pos are read
   const int start = first_visible_key(pos, window);   // window < 0: chunks of -window
@@ -169,7 +174,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   u32x4_t qf[KSTEPS];
   {
     const bool valid = col < G;
-    const bf16_t* qr = q + (static_cast<size_t>(t) * H + static_cast<size_t>(kvh) * G + (valid ? col : 0)) * DH;
+    const bf16_t* qr = q + (static_cast<size_t>(t) * H + head0 + (valid ? col : 0)) * DH;
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
       const int d = st * 32 + quad * 8;
@@ -278,7 +283,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_kernel(
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
-  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e,
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, head0 + col, H, quad, nsplit, split, scale_log2e,
               sinks);
 }
 
@@ -326,9 +331,14 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   // workgroup of the sequence's eight from pair to pair, or a few XCDs would carry all the work.
   const int split = share_tiles != nullptr ? static_cast<int>((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x)
                                            : static_cast<int>(blockIdx.x);
-  const int kvh = blockIdx.y;
+  // More than 16 query heads a KV head run as several waves of up to 16 columns each: blockIdx.y counts
+  // (KV head, group of 16 heads).
+  const int heads_per_kv = H / KVH;
+  const int column_groups = (heads_per_kv + 15) / 16;
+  const int kvh = static_cast<int>(blockIdx.y) / column_groups;
+  const int head0 = kvh * heads_per_kv + (static_cast<int>(blockIdx.y) % column_groups) * 16;   // column 0's query head
   const int s = seq_ids ? seq_ids[blockIdx.z] : blockIdx.z;
-  const int G = H / KVH;
+  const int G = min(16, kvh * heads_per_kv + heads_per_kv - head0);                          // this wave's columns
   const int t = query_start[s];
   const int pos = context_lens[s] - 1;
   const int start = first_visible_key(pos, window);   // window < 0: chunks of -window
@@ -347,7 +357,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   if (share_tiles != nullptr && tile_begin >= tile_end) {
     // An empty share leaves at once: a maximum of -inf gives it no weight, and the merge does not read the rest.
     if (quad == 0 && col < G) {
-      const size_t slot = (static_cast<size_t>(blockIdx.z) * H + kvh * G + col) * nsplit + split;
+      const size_t slot = (static_cast<size_t>(blockIdx.z) * H + head0 + col) * nsplit + split;
       part_ml[slot * 2] = -INFINITY;
       part_ml[slot * 2 + 1] = 0.f;
     }
@@ -367,7 +377,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   if constexpr (PREPARE) {
   } else {
     const bool valid = col < G;
-    const bf16_t* qr = q + (static_cast<size_t>(t) * H + static_cast<size_t>(kvh) * G + (valid ? col : 0)) * DH;
+    const bf16_t* qr = q + (static_cast<size_t>(t) * H + head0 + (valid ? col : 0)) * DH;
 #pragma unroll
     for (int st = 0; st < KSTEPS; ++st) {
       const int d = st * 32 + quad * 8;
@@ -436,7 +446,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     // the group read its last head again) and, in the wave that takes the newest token, its key (the lanes
     // of even heads-worth) or value (odd), 4 + 4 elements a lane like a query's.
     const int g_first = lane / LPH;
-    const float* q_in = row + (static_cast<size_t>(kvh) * G + min(g_first, G - 1)) * DH;
+    const float* q_in = row + (static_cast<size_t>(head0) + min(g_first, G - 1)) * DH;
     qk_f4_t qa = load4_planes(q_in + p0, src.plane_stride, src.planes);
     qk_f4_t qb = load4_planes(q_in + HALF + p0, src.plane_stride, src.planes);
     qk_f4_t na = {0.f, 0.f, 0.f, 0.f}, nb = na;
@@ -480,7 +490,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
     for (int g0 = HEADS_AT_ONCE; g0 < G; g0 += HEADS_AT_ONCE) {
       const int g = g0 + lane / LPH;
       if (g < G) {
-        const float* in = row + (static_cast<size_t>(kvh) * G + g) * DH;
+        const float* in = row + (static_cast<size_t>(head0) + g) * DH;
         qk_f4_t a = load4_planes(in + p0, src.plane_stride, src.planes);
         qk_f4_t b = load4_planes(in + HALF + p0, src.plane_stride, src.planes);
         if (src.q_weight != nullptr) qk_head_norm<LPH>(a, b, src.q_weight, src.eps, p0);
@@ -567,7 +577,7 @@ __global__ __launch_bounds__(TIE_WAVE) void attention_decode_ring_kernel(
   l += __shfl_xor(l, 16, TIE_WAVE);
   l += __shfl_xor(l, 32, TIE_WAVE);
   if (col >= G) return;
-  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, kvh * G + col, H, quad, nsplit, split, scale_log2e,
+  store_share(acc, m, l, out, part_o, part_ml, t, blockIdx.z, head0 + col, H, quad, nsplit, split, scale_log2e,
               sinks);
 }
 
@@ -585,7 +595,9 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
                          int depth, const float* sinks, hipStream_t stream, int keep = 0) {
   // kept first positions go beside a window, with uncapped scores and queries that come ready
   if (keep < 0 || (keep > 0 && (window <= 0 || softcap > 0.f || src != nullptr))) return TIE_BAD_ARGUMENT;
-  if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH > 65535 || H % KVH != 0 || H / KVH > 16 ||
+  const int column_groups = KVH > 0 ? (H / KVH + 15) / 16 : 1;    // waves of up to 16 query heads a KV head
+  if (num_seqs <= 0 || num_seqs > 65535 || H <= 0 || KVH <= 0 || KVH * column_groups > 65535 || H % KVH != 0 ||
+      (src != nullptr && H / KVH > 16) ||
       block_size < 4 || (block_size & (block_size - 1)) != 0 || max_blocks <= 0 || nsplit <= 0 ||
       nsplit > MERGE_MAX_SPLITS || depth < 0 || depth > 4 || (depth > 1 && block_size < 16) ||
       !(scale > 0.f))   // the running maximum is kept on unscaled scores
@@ -596,7 +608,7 @@ static int launch_decode(const bf16_t* q, const QkSource* src, bf16_t* k_cache, 
   if (depth == 0) depth = block_size < 16 ? 1 : (nsplit == 1 ? 4 : 3);
   if (src != nullptr && (depth < 2 || !PREPARE_HEAD_DIM)) return TIE_BAD_ARGUMENT;
   if (share_tiles != nullptr && (depth < 2 || nsplit == 1)) return TIE_BAD_ARGUMENT;   // the ring kernel's, with a merge
-  const dim3 grid(nsplit, KVH, num_seqs);
+  const dim3 grid(nsplit, KVH * column_groups, num_seqs);
   const int block_shift = __builtin_ctz(block_size);
   const float scale_log2e = scale * 1.44269504088896340736f;
   const float cap = softcap > 0.f ? softcap / scale : 0.f;   // softcap * tanh(scale s / softcap) = scale * cap tanh(s / cap)

@@ -1362,9 +1362,9 @@ def attention_decode_bf16(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         raise InvalidArgument("attention_decode_bf16 takes bfloat16 queries, cache and output")
     if q.shape[1] != H * Dh or out.shape != q.shape:
         raise InvalidArgument(f"attention: q {list(q.shape)} / out {list(out.shape)} do not fit {H} heads of {Dh}")
-    if Dh not in MFMA_HEAD_DIMS or H % KVH or H // KVH > 16 or not mfma_block_size(bs):
-        raise InvalidArgument(f"attention_decode_bf16 takes head sizes in steps of 16 up to 256, at most 16 query heads "
-                              f"a KV head and block sizes 4, 8, 16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
+    if Dh not in MFMA_HEAD_DIMS or H % KVH or not mfma_block_size(bs):
+        raise InvalidArgument(f"attention_decode_bf16 takes head sizes in steps of 16 up to 256 and block sizes 4, 8, "
+                              f"16, ...; got head_dim {Dh}, {H}/{KVH} heads, block {bs}")
     _i32(query_start, "query_start")
     _i32(context_lens, "context_lens")
     _i32(block_tables, "block tables")
@@ -1568,7 +1568,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if keep_first and softcap:
         fast = False           # kept first positions beside capped scores: the generic kernel alone takes both
     reach = (window + keep_first if window else None) or chunk      # the most keys a query reads: what the shares of a sequence's keys are planned by
-    if fast and batch.all_decode and num_heads // KVH <= 16:
+    if fast and batch.all_decode:          # more than 16 query heads a KV head: several waves of 16 columns
         S = batch.num_seqs
         nsplit, share_tiles = step_key_shares(step, S, KVH, batch.plan_context, bs)
         part_o = part_ml = None
@@ -1579,11 +1579,6 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                               S, num_heads, scale, window, nsplit, part_o, part_ml, share_tiles=share_tiles,
                               softcap=softcap, chunk=chunk, sinks=sinks, keep_first=keep_first)
         return
-    if fast and batch.all_decode:
-        # Single tokens of more than 16 query heads a KV head: the decode kernel does not take them, and the work
-        # lists of the prompt kernel below are built on the host and live only as long as the step, which a
-        # recorded decode step would outlive. The generic kernel reads the step on the device.
-        fast = False
     if fast:
         # A mixed step: sequences that bring one decoded token go to the decode kernel (their keys are
         # split over many waves), the prompt portions to the prefill kernel. Built once a step.
@@ -1592,7 +1587,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         work = batch.memo.get(key)
         if work is None:
             new = batch.host_new_tokens
-            single = [s for s, n in enumerate(new) if n == 1] if G <= 16 else []
+            single = [s for s, n in enumerate(new) if n == 1]
             if len(single) == len(new):
                 single = []                                   # nothing but single rows and yet not a decode step
             elif len(single) * KVH * -(-G // min(G, 4)) <= SINGLE_ROWS_RIDE_ALONG:
