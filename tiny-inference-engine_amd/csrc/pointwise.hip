@@ -5,13 +5,22 @@
 //                  still owed to it (a product cut along K) are added first, in plane order, and the sum is
 //                  written back, so the pass that reads the stream anyway also settles it. Rows can be gathered
 //                  (the head norms only the wanted rows). `plain` leaves out the function: out = x in the
-//                  output's type, for a consumer that reads the stream itself.
+//                  output's type, for a consumer that reads the stream itself. Float32 rows out take the
+//                  library's tanhf; rows that are rounded to bfloat16 anyway take tanh on the hardware's 2^x and
+//                  reciprocal (float32 arithmetic, absolute error of a few 1e-7).
 //   token_gate     out[t][j] = gelu_tanh(gate[t][j]) * table[token[t]][first + j]: a per-token vector out of a
 //                  table that all layers share, each with a range of columns of its own, multiplied into a gate
 //                  the layer computed from the stream.
 #include "common.h"
 
 #include <math.h>
+
+template <typename TO>
+__device__ __forceinline__ float tanh_for(float x);
+template <>
+__device__ __forceinline__ float tanh_for<float>(float x) { return tanhf(x); }
+template <>
+__device__ __forceinline__ float tanh_for<bf16_t>(float x) { return tanh_fast(x); }
 
 template <typename TO, bool PLAIN>
 __global__ void dynamic_tanh_kernel(float* __restrict__ x, const float* __restrict__ partials, size_t plane_stride,
@@ -35,7 +44,7 @@ __global__ void dynamic_tanh_kernel(float* __restrict__ x, const float* __restri
       float y[4] = {v.x, v.y, v.z, v.w};
       if (!PLAIN) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) y[j] = fmaf(tanhf(a * y[j]), w[i + j], b[i + j]);
+        for (int j = 0; j < 4; ++j) y[j] = fmaf(tanh_for<TO>(a * y[j]), w[i + j], b[i + j]);
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) store_from_float(out + r * n + i + j, y[j]);
@@ -46,7 +55,7 @@ __global__ void dynamic_tanh_kernel(float* __restrict__ x, const float* __restri
           for (int p = 0; p < planes; ++p) v += partials[p * plane_stride + at + j];
           x[at + j] = v;
         }
-        store_from_float(out + r * n + i + j, PLAIN ? v : fmaf(tanhf(a * v), w[i + j], b[i + j]));
+        store_from_float(out + r * n + i + j, PLAIN ? v : fmaf(tanh_for<TO>(a * v), w[i + j], b[i + j]));
       }
     }
   }
