@@ -3,7 +3,8 @@
 //
 // One wave handles one (sequence, KV head, split of the keys). The G = H / KVH query heads that
 // share the KV head are the 16 columns of the MFMA tiles (columns >= G are zeros), so keys and
-// values are read once for the whole group. Per 32 keys:
+// values are read once for the whole group; more than 16 heads a KV head are several waves of up to
+// 16 columns each. Per 32 keys:
 //
 //   S^T[key, g] = K[key, :] . Q[g, :]      A = K rows (16 bytes a lane, straight from the cache),
 //                                          B = Q (held in registers)          2 x HEAD_DIM/32 MFMAs
