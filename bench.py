@@ -167,7 +167,7 @@ ZOVUDRA_SIZES = {
 def zovudra_config(size):
     dense = {"kind": "dense", "ff": size["ff"]}
     moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "shared": {"ff": size["shared_ff"]},
-           "router": {"experts": size["experts"], "top": size["top"], "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+           "router": {"experts": size["experts"], "top": size["top"], "scale": 2.0, "groups": {"count": 4, "keep": 2}}}
     attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
                  "scale": size["dim"] ** -0.5, "mask": {"size": size["window"], "keep_first": size["keep_first"]},
                  "rot": {"dims": size["dim"], "base": 500000.0,

@@ -83,7 +83,7 @@ C = {
     "architecture": "Zovudra", "vocab": 333, "width": 100, "norm": {"eps": 1e-4}, "embedding": {"scale": 0.5},
     "token_side": {"dim": 6},
     "layers": [
-        {**_latent(5, 10, 6, 7, 13, 11, 0.3, None, _rot(6, 30.0)), "mlp": _moe(9, 5, 2, 2.5, None, 5)},
+        {**_latent(5, 10, 6, 7, 13, 11, 0.3, None, _rot(6, 30.0)), "mlp": _moe(9, 5, 2, 2.25, None, 5)},
         {**_attention(3, 3, 10, 7, 0.28, 11, 2, _rot(6, 70.0, (5.0, 0.5, 2.0, 16))), "mlp": _dense(50)},
     ],
 }
@@ -98,10 +98,10 @@ E = {
     "architecture": "Zovudra", "vocab": 150, "width": 256, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.5},
     "token_side": {"dim": 32},
     "layers": [
-        {**_attention(4, 2, 128, 128, 0.09, 64, 4, _rot(128, 250000.0, (4.0, 1.0, 4.0, 128))),
+        {**_attention(4, 2, 128, 128, 0.09, 64, 4, _rot(128, 400000.0, (6.0, 1.0, 4.0, 128))),
          "mlp": _moe(64, 8, 2, 2.0, (2, 1), 128)},
         {**_latent(4, 64, 32, 64, 96, 48, 0.1, 40, _rot(32, 10000.0)), "mlp": _dense(128)},
-        {**_attention(4, 2, 128, 128, 0.09, 64, 4, _rot(128, 250000.0, (4.0, 1.0, 4.0, 128))), "mlp": _dense(96)},
+        {**_attention(4, 2, 128, 128, 0.09, 64, 4, _rot(128, 400000.0, (6.0, 1.0, 4.0, 128))), "mlp": _dense(96)},
     ],
 }
 CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E}
