@@ -226,6 +226,13 @@ class StepContext:
         self._late = None
         return payload
 
+    def run_late(self) -> None:
+        """Runs a pass a block left for the one behind it, if any (for a block that does not merge such passes)."""
+        if self._late is not None:
+            _, run, payload = self._late
+            self._late = None
+            run(payload)
+
     def launch_pending(self) -> None:
         """Launches a product left pending the ordinary way (it may leave planes of partial sums owed in turn)."""
         if self._pending is not None:
@@ -256,10 +263,7 @@ class StepContext:
         return None
 
     def settle(self) -> None:
-        if self._late is not None:
-            _, run, payload = self._late
-            self._late = None
-            run(payload)
+        self.run_late()
         self.launch_pending()
         if self._owed is not None:
             from .. import kernels

@@ -108,8 +108,7 @@ class TokenSideBlock(PreNormBlock):
             rows = x
         else:
             # the stream in the products' type, in the pass that adds what the feed-forward still owes it
-            if ctx._late is not None:
-                ctx.settle()
+            ctx.run_late()
             owed = ctx.take_owed(x)
             rows = ctx.scratch("token_side.rows", (T, self.hidden), ctx.act_dtype)
             ctx.set_row_scale(rows, None)
